@@ -1,0 +1,297 @@
+// Attention over a cached low-rank latent (one per token, shared by all heads) with a rotated key part shared by all
+// heads and a per-head sink logit in the softmax's denominator.
+//
+// The cache of a token is c [rank] (normalised latent) and kr [rot] (rotated key part).  A head's key is W_uk c and
+// its value W_uv c; neither is ever made.  Instead the query is taken into the latent's space,
+//     qa_h = W_uk,h^T q_h          (q_h the head's unrotated part),
+// so that score(h, j) = scale * (qa_h . c_j + qr_h . kr_j), and the weighted sum runs over the latents themselves,
+//     u_h = sum_j p(h, j) c_j,     value_h = W_uv,h u_h.
+// Every head reads the same cached row: one staged tile of keys serves all heads of a block.
+// The sink: a logit s_h with no key and no value; it enters the running maximum and the denominator once
+// (running state starts at maximum s_h, sum 1, result 0).
+#include "common.h"
+#include "partials.h"
+
+// ---------------------------------------------------------------------------------------------------------------
+// Step 1 of the mixer, after the stacked down products x = [W_dq h ; W_dkv h] (q_rank + rank + rot columns):
+//   cq = x[:q_rank] / sqrt(mean(.^2) + eps) * wq                     -> cq_out (T)
+//   c  = x[q_rank : q_rank + rank] / sqrt(mean(.^2) + eps) * wc      -> latent cache at the row's slot
+//   kr = rotate(x[q_rank + rank :], position)                        -> rope cache at the row's slot
+// Rotation of a vector of `rot` elements: element i pairs with i + rot / 2, angle position * freq[i].
+template <typename TD, typename T>
+__global__ void latent_prepare_kernel(const TD* __restrict__ x, int splits, size_t split_stride, const float* __restrict__ wq,
+                                      const float* __restrict__ wc, const float* __restrict__ freq,
+                                      const int* __restrict__ positions, const int* __restrict__ slots, T* __restrict__ cq_out,
+                                      T* __restrict__ latent, T* __restrict__ rope, int q_rank, int rank, int rot, float eps) {
+  __shared__ float scratch[16];
+  const int n = blockIdx.x, total = q_rank + rank + rot;
+  const size_t at = (size_t)n * total;
+  float sq = 0.f, sc = 0.f;
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x) { const float v = parts_sum(x, at + i, splits, split_stride); sq += v * v; }
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) { const float v = parts_sum(x, at + q_rank + i, splits, split_stride); sc += v * v; }
+  sq = block_sum(sq, scratch);
+  sc = block_sum(sc, scratch);
+  const float rq = 1.f / sqrtf(sq / (float)q_rank + eps), rc = 1.f / sqrtf(sc / (float)rank + eps);
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x)
+    st(cq_out + (size_t)n * q_rank + i, parts_sum(x, at + i, splits, split_stride) * rq * wq[i]);
+  if (!slots) return;
+  const size_t slot = (size_t)slots[n];
+  for (int i = threadIdx.x; i < rank; i += blockDim.x)
+    st(latent + slot * rank + i, parts_sum(x, at + q_rank + i, splits, split_stride) * rc * wc[i]);
+  const int half = rot / 2;
+  const float p = (float)positions[n];
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float u = parts_sum(x, at + q_rank + rank + i, splits, split_stride);
+    const float v = parts_sum(x, at + q_rank + rank + half + i, splits, split_stride);
+    float sn, cs;
+    sincosf(p * freq[i], &sn, &cs);
+    st(rope + slot * rot + i, u * cs - v * sn);
+    st(rope + slot * rot + half + i, v * cs + u * sn);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// A product per head: out[n, h, o] = sum_k W[h, k, o] x[n, h, k]   (W "k-major": the outputs of one k side by side).
+// x: row stride x_row, head stride x_head (elements); out likewise.  A block takes ROWS rows of one head and 256
+// outputs; x passes through LDS, every W element is read once a block.
+template <typename TX, typename TW, typename TO, int ROWS>
+__global__ void head_product_kernel(const TX* __restrict__ x, int x_row, int x_head, const TW* __restrict__ w,
+                                    TO* __restrict__ out, int out_row, int out_head, int n_rows, int k_dim, int o_dim) {
+  extern __shared__ float xs[];                       // [ROWS][k_dim]
+  const int row0 = blockIdx.x * ROWS, h = blockIdx.y, o = blockIdx.z * blockDim.x + threadIdx.x;
+  for (int idx = threadIdx.x; idx < ROWS * k_dim; idx += blockDim.x) {
+    const int r = idx / k_dim, k = idx - r * k_dim;
+    xs[idx] = row0 + r < n_rows ? ld(x + (size_t)(row0 + r) * x_row + (size_t)h * x_head + k) : 0.f;
+  }
+  __syncthreads();
+  if (o >= o_dim) return;
+  float acc[ROWS];
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r) acc[r] = 0.f;
+  const TW* wh = w + (size_t)h * k_dim * o_dim + o;
+  for (int k = 0; k < k_dim; ++k) {
+    const float wv = ld(wh + (size_t)k * o_dim);
+#pragma unroll
+    for (int r = 0; r < ROWS; ++r) acc[r] += wv * xs[r * k_dim + k];
+  }
+#pragma unroll
+  for (int r = 0; r < ROWS; ++r)
+    if (row0 + r < n_rows) st(out + (size_t)(row0 + r) * out_row + (size_t)h * out_head + o, acc[r]);
+}
+
+// The rotated tail of every head's query: out[n, h, i] = rotate(q[n, h, offset + i], position), i < rot.
+template <typename TX>
+__global__ void rotate_tail_kernel(const TX* __restrict__ q, int q_row, int q_head, int offset, const float* __restrict__ freq,
+                                   const int* __restrict__ positions, float* __restrict__ out, int out_row, int out_head,
+                                   int out_offset, int rot) {
+  const int n = blockIdx.x, h = blockIdx.y, half = rot / 2;
+  const float p = (float)positions[n];
+  const TX* src = q + (size_t)n * q_row + (size_t)h * q_head + offset;
+  float* dst = out + (size_t)n * out_row + (size_t)h * out_head + out_offset;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float u = ld(src + i), v = ld(src + half + i);
+    float sn, cs;
+    sincosf(p * freq[i], &sn, &cs);
+    dst[i] = u * cs - v * sn;
+    dst[half + i] = v * cs + u * sn;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The general kernel: one block per (row, group of heads), any sizes, float32 arithmetic on the vector units.
+//   Q [N, H, D] float32, D = rank + rot (qa then the rotated part); caches latent [slots, rank], rope [slots, rot] (TC);
+//   out [N, H, rank] float32 = sum_j p(h, j) c_j.
+// Keys come in tiles of KT (<= 64) rows staged in LDS as float32; a wave makes one head's softmax step with a lane
+// per key; a thread owns up to ACC elements (h, c) of the group's results.
+#define LA_THREADS 256
+#define LA_ACC 16
+template <typename TC>
+__global__ void __launch_bounds__(LA_THREADS)
+latent_attention_kernel(const float* __restrict__ q, const TC* __restrict__ latent, const TC* __restrict__ rope,
+                        const int* __restrict__ tables, int table_stride, const int* __restrict__ row_seq,
+                        const int* __restrict__ positions, const float* __restrict__ sink, float* __restrict__ out,
+                        int heads, int group, int rank, int rot, int page_size, int kt, float scale) {
+  extern __shared__ float lds[];
+  const int d = rank + rot, pad = d + 1;
+  float* qs = lds;                                   // [group][d]
+  float* ks = qs + group * d;                        // [kt][pad]
+  float* ps = ks + kt * pad;                         // [group][kt]
+  float* top = ps + group * kt;                      // [group]
+  float* den = top + group;                          // [group]
+  float* shrink = den + group;                       // [group]
+  const int n = blockIdx.x, h0 = blockIdx.y * group;
+  const int live = min(group, heads - h0);
+  const int position = positions[n];
+  const int* table = tables + (size_t)row_seq[n] * table_stride;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  for (int idx = tid; idx < live * d; idx += LA_THREADS) qs[idx] = q[((size_t)n * heads + h0) * d + idx];
+  if (tid < live) { top[tid] = sink ? sink[h0 + tid] : -INFINITY; den[tid] = sink ? 1.f : 0.f; }
+  float acc[LA_ACC];
+#pragma unroll
+  for (int a = 0; a < LA_ACC; ++a) acc[a] = 0.f;
+  const int owned = live * rank;
+
+  for (int j0 = 0; j0 <= position; j0 += kt) {
+    const int keys = min(kt, position + 1 - j0);
+    __syncthreads();                                 // the last tile's reads are done (and qs / top / den are written)
+    for (int idx = tid; idx < keys * d; idx += LA_THREADS) {
+      const int j = idx / d, i = idx - j * d;
+      const int key = j0 + j;
+      const size_t slot = (size_t)table[key / page_size] * page_size + key % page_size;
+      ks[j * pad + i] = i < rank ? ld(latent + slot * rank + i) : ld(rope + slot * rot + (i - rank));
+    }
+    __syncthreads();
+    for (int pair = tid; pair < live * kt; pair += LA_THREADS) {
+      const int h = pair / kt, j = pair - h * kt;
+      float s = -INFINITY;
+      if (j < keys) {
+        const float* qh = qs + h * d;
+        const float* kj = ks + j * pad;
+        float dot = 0.f;
+        for (int i = 0; i < d; ++i) dot += qh[i] * kj[i];
+        s = dot * scale;
+      }
+      ps[pair] = s;
+    }
+    __syncthreads();
+    for (int h = wave; h < live; h += LA_THREADS / 64) {
+      const float s = lane < kt ? ps[h * kt + lane] : -INFINITY;
+      const float old = top[h];
+      const float now = fmaxf(old, wave_max(s));
+      const float p = (lane < keys && now > -INFINITY) ? expf(s - now) : 0.f;
+      const float total = wave_sum(p);
+      if (lane < kt) ps[h * kt + lane] = p;
+      if (lane == 0) {
+        const float f = now > -INFINITY ? expf(old - now) : 1.f;
+        shrink[h] = f;
+        den[h] = den[h] * f + total;
+        top[h] = now;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int a = 0; a < LA_ACC; ++a) {
+      const int e = tid + a * LA_THREADS;
+      if (e < owned) {
+        const int h = e / rank, c = e - h * rank;
+        float v = acc[a] * shrink[h];
+        const float* ph = ps + h * kt;
+        for (int j = 0; j < keys; ++j) v += ph[j] * ks[j * pad + c];
+        acc[a] = v;
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int a = 0; a < LA_ACC; ++a) {
+    const int e = tid + a * LA_THREADS;
+    if (e < owned) {
+      const int h = e / rank, c = e - h * rank;
+      out[((size_t)n * heads + h0 + h) * rank + c] = acc[a] / den[h];
+    }
+  }
+}
+
+// Heads a block of the general kernel takes, and the keys of a staged tile, for these sizes.
+static void latent_plan(int heads, int rank, int rot, int* group, int* kt, size_t* lds) {
+  const int d = rank + rot;
+  int g = LA_ACC * LA_THREADS / rank;
+  if (g > heads) g = heads;
+  while (g > 1 && (size_t)g * d * 4 > 24 * 1024) --g;
+  int t = 64;
+  while (t > 1 && (size_t)t * (d + 1) * 4 > 32 * 1024) t /= 2;
+  *group = g;
+  *kt = t;
+  *lds = ((size_t)g * d + (size_t)t * (d + 1) + (size_t)g * t + 3 * (size_t)g) * sizeof(float);
+}
+
+extern "C" {
+
+int qil_latent_prepare(const void* x, int x_dtype, int splits, const float* wq, const float* wc, const float* freq,
+                       const int* positions, const int* slots, void* cq_out, void* latent, void* rope, int n, int q_rank,
+                       int rank, int rot, float eps, int dtype, hipStream_t s) {
+  if (n == 0) return 0;
+  if (q_rank < 1 || rank < 1 || rot < 2 || rot % 2 || splits < 1 || (x_dtype == QIL_BF16 && splits != 1)) return -1;
+  const size_t stride = (size_t)n * (q_rank + rank + rot);
+#define QIL_LP(TD, T)                                                                                               \
+  hipLaunchKernelGGL((latent_prepare_kernel<TD, T>), dim3(n), dim3(256), 0, s, (const TD*)x, splits, stride, wq, wc, \
+                     freq, positions, slots, (T*)cq_out, (T*)latent, (T*)rope, q_rank, rank, rot, eps)
+  if (dtype == QIL_F32) {
+    if (x_dtype != QIL_F32) return -1;
+    QIL_LP(float, float);
+  } else if (x_dtype == QIL_F32) {
+    QIL_LP(float, bf16_t);
+  } else {
+    QIL_LP(bf16_t, bf16_t);
+  }
+#undef QIL_LP
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+// out[n, h, o] = sum_k w[h, k, o] x[n, h, k]; x_dtype / w_dtype / out_dtype element codes; strides in elements.
+// Combinations: all float32; x bfloat16, w bfloat16, out float32; x float32, w bfloat16, out bfloat16.
+int qil_head_product(const void* x, int x_dtype, int x_row, int x_head, const void* w, int w_dtype, void* out,
+                     int out_dtype, int out_row, int out_head, int n, int heads, int k_dim, int o_dim, hipStream_t s) {
+  if (n == 0 || heads == 0 || o_dim == 0) return 0;
+  if (k_dim < 1) return -1;
+  const int rows = 8;
+  const size_t lds = (size_t)rows * k_dim * sizeof(float);
+  if (lds > 64 * 1024) return -1;
+  const int threads = o_dim >= 256 ? 256 : (o_dim + 63) / 64 * 64;
+  dim3 grid((n + rows - 1) / rows, heads, (o_dim + threads - 1) / threads);
+#define QIL_HP(TX, TW, TO)                                                                                          \
+  hipLaunchKernelGGL((head_product_kernel<TX, TW, TO, 8>), grid, dim3(threads), lds, s, (const TX*)x, x_row, x_head, \
+                     (const TW*)w, (TO*)out, out_row, out_head, n, k_dim, o_dim)
+  if (x_dtype == QIL_F32 && w_dtype == QIL_F32 && out_dtype == QIL_F32) QIL_HP(float, float, float);
+  else if (x_dtype == QIL_BF16 && w_dtype == QIL_BF16 && out_dtype == QIL_F32) QIL_HP(bf16_t, bf16_t, float);
+  else if (x_dtype == QIL_F32 && w_dtype == QIL_BF16 && out_dtype == QIL_BF16) QIL_HP(float, bf16_t, bf16_t);
+  else return -1;
+#undef QIL_HP
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+// out[n, h, out_offset + i] = rotate(q[n, h, offset + i], positions[n]) for i < rot; out float32.
+int qil_rotate_tail(const void* q, int q_dtype, int q_row, int q_head, int offset, const float* freq, const int* positions,
+                    float* out, int out_row, int out_head, int out_offset, int n, int heads, int rot, hipStream_t s) {
+  if (n == 0 || heads == 0) return 0;
+  if (rot < 2 || rot % 2) return -1;
+  if (q_dtype == QIL_F32)
+    hipLaunchKernelGGL(rotate_tail_kernel<float>, dim3(n, heads), dim3(64), 0, s, (const float*)q, q_row, q_head, offset,
+                       freq, positions, out, out_row, out_head, out_offset, rot);
+  else
+    hipLaunchKernelGGL(rotate_tail_kernel<bf16_t>, dim3(n, heads), dim3(64), 0, s, (const bf16_t*)q, q_row, q_head, offset,
+                       freq, positions, out, out_row, out_head, out_offset, rot);
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+// Whether the general kernel takes these sizes.
+int qil_latent_attention_takes(int heads, int rank, int rot) {
+  if (heads < 1 || rank < 1 || rot < 0 || rank > LA_ACC * LA_THREADS) return 0;
+  int group, kt;
+  size_t lds;
+  latent_plan(heads, rank, rot, &group, &kt, &lds);
+  return group >= 1 && kt >= 1 && (size_t)group * (rank + rot) * 4 <= 24 * 1024 && lds <= 64 * 1024;
+}
+
+int qil_latent_attention(const float* q, const void* latent, const void* rope, const int* tables, int table_stride,
+                         const int* row_seq, const int* positions, const float* sink, float* out, int n, int heads,
+                         int rank, int rot, int page_size, float scale, int cache_dtype, hipStream_t s) {
+  if (n == 0) return 0;
+  if (!qil_latent_attention_takes(heads, rank, rot) || page_size < 1) return -1;
+  int group, kt;
+  size_t lds;
+  latent_plan(heads, rank, rot, &group, &kt, &lds);
+  dim3 grid(n, (heads + group - 1) / group);
+  if (cache_dtype == QIL_F32)
+    hipLaunchKernelGGL(latent_attention_kernel<float>, grid, dim3(LA_THREADS), lds, s, q, (const float*)latent,
+                       (const float*)rope, tables, table_stride, row_seq, positions, sink, out, heads, group, rank, rot,
+                       page_size, kt, scale);
+  else
+    hipLaunchKernelGGL(latent_attention_kernel<bf16_t>, grid, dim3(LA_THREADS), lds, s, q, (const bf16_t*)latent,
+                       (const bf16_t*)rope, tables, table_stride, row_seq, positions, sink, out, heads, group, rank, rot,
+                       page_size, kt, scale);
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+}  // extern "C"

@@ -21,6 +21,7 @@ from .step import ModelRunner
 
 PAGE_SIZE = 16
 ROUND_TO = 64          # a live request's token count is rounded up to this (or to a page, if larger)
+MAX_REQUESTS = 4       # requests that are live at any time: state slots are made for this many
 
 
 def pages_for_budget(max_tokens, page_size):
@@ -29,7 +30,7 @@ def pages_for_budget(max_tokens, page_size):
 
 
 class Replay:
-    def __init__(self, model, *, max_tokens, page_size=PAGE_SIZE, max_requests=64):
+    def __init__(self, model, *, max_tokens, page_size=PAGE_SIZE, max_requests=MAX_REQUESTS):
         self.runner = ModelRunner(model, num_pages=pages_for_budget(max_tokens, page_size), page_size=page_size,
                                   max_requests=max_requests)
 

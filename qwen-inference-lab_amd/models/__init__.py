@@ -1,2 +1,3 @@
 """Built-in architectures; importing this package registers them."""
 from . import qwen3  # noqa: F401
+from . import fubapel  # noqa: F401

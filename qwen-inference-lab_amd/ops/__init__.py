@@ -406,8 +406,8 @@ def interleave_gate_up(gate, up):
     return torch.stack((gate.view(inner // 16, 16, k), up.view(inner // 16, 16, k)), dim=1).reshape(2 * inner, k).contiguous()
 
 
-def gated_linear(x, weight, out_dtype=None, interleaved=False, lazy=False):
-    """silu(x @ gate^T) * (x @ up^T) -> [N, I], with ``weight`` the [2 I, K] matrix of both: the gate rows stacked
+def gated_linear(x, weight, out_dtype=None, interleaved=False, lazy=False, activation='silu', limit=0.0, alpha=1.0):
+    """act(x @ gate^T, x @ up^T) -> [N, I] (``activation``: a name of ``GATE_FUNCTIONS``; silu(gate) * up unless said), with ``weight`` the [2 I, K] matrix of both: the gate rows stacked
     before the up rows, or (``interleaved``) both in turns of 16 rows, which the kernels read faster.
 
     One kernel when a fused kernel takes the sizes (bfloat16; up to 16 rows, or up to 256 rows of an interleaved
@@ -424,6 +424,9 @@ def gated_linear(x, weight, out_dtype=None, interleaved=False, lazy=False):
         raise ValueError(f'gated_linear: x {tuple(x.shape)}, weight {tuple(weight.shape)}')
     out_dtype = out_dtype or x.dtype
     lib = library.load()
+    if activation != 'silu':                       # the product, then the activation kernel
+        return gated_act(linear(x, weight, None, partials=True), out_dtype, activation=activation, limit=limit, alpha=alpha,
+                         interleaved=interleaved)
     # 17 to 256 rows of an interleaved matrix: the 32 x 32 tile kernel where it takes the sizes (measured against the
     # staged 16 x 16 kernel with the same epilogue at 17 to 64 rows: 37 to 38 us against 38 to 43 at Qwen3-8B sizes,
     # 73 to 85 against 87 to 102 at 14B sizes)
@@ -746,3 +749,215 @@ def sample(logits, temperatures, seeds, counters, out=None):
     _check(lib.qil_sample(_ptr(logits), _ptr(temperatures), _ptr(seeds), _ptr(counters), _ptr(tokens), _ptr(finite),
                           _ptr(workspace), m, vocab, _stream()), 'sample')
     return tokens, finite
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Norms with a scaled residual add; gate functions by name
+def add_norm(stream, delta, weight, eps, out_dtype, *, centre, delta_scale=1.0):
+    """stream += delta_scale * delta (in place, float32; skipped if delta is None); returns the norm of the sum as
+    out_dtype: layer norm without a bias (``centre``: the mean is removed, the variance is that of the centred row)
+    or RMS norm, times ``weight``, rounded once.  ``delta``: tensor of ``out_dtype`` [N, H] or Partials."""
+    n, width = stream.shape
+    _require(stream, 'stream', torch.float32)
+    _require(weight, 'weight', torch.float32, (width,))
+    pointer, code, splits = (None, _code(out_dtype), 1) if delta is None else _operand(delta, 'delta', out_dtype, (n, width))
+    out = torch.empty((n, width), dtype=out_dtype, device=stream.device)
+    _check(library.load().qil_add_norm(_ptr(stream), pointer, code, splits, n, float(delta_scale), None, _ptr(weight),
+                                       _ptr(out), n, width, float(eps), 1, int(bool(centre)), _code(out_dtype), _stream()),
+           'add_norm')
+    return out
+
+
+def rows_norm(stream, delta, rows, weight, eps, out_dtype, *, centre, delta_scale=1.0):
+    """``add_norm`` of the selected rows only, [len(rows), H]; stream is left as it is."""
+    n, width = stream.shape
+    _require(stream, 'stream', torch.float32)
+    _require(weight, 'weight', torch.float32, (width,))
+    _require(rows, 'rows', torch.int32)
+    pointer, code, splits = (None, _code(out_dtype), 1) if delta is None else _operand(delta, 'delta', out_dtype, (n, width))
+    out = torch.empty((rows.shape[0], width), dtype=out_dtype, device=stream.device)
+    _check(library.load().qil_add_norm(_ptr(stream), pointer, code, splits, n, float(delta_scale), _ptr(rows), _ptr(weight),
+                                       _ptr(out), rows.shape[0], width, float(eps), 0, int(bool(centre)), _code(out_dtype),
+                                       _stream()), 'rows_norm')
+    return out
+
+
+# Gate functions of gated feed-forwards: name -> code of the kernels.  'silu': silu(g) * u.  'clamped_swish' (with a
+# limit L and a slope a): g' = min(g, L), u' = clamp(u, -L, L), g' * sigmoid(a g') * (u' + 1).
+GATE_FUNCTIONS = {'silu': 0, 'clamped_swish': 1}
+
+
+def gated_act(gate_up, out_dtype, *, activation, limit=0.0, alpha=1.0, interleaved=False):
+    """[N, 2 I] (tensor of the model's type or Partials) -> act(gate, up), [N, I], for any gate function of
+    ``GATE_FUNCTIONS``.  The gate columns come first, or (``interleaved``) gate and up columns come in turns of 16."""
+    n, both = gate_up.shape
+    if both % 2 or (interleaved and both % 32):
+        raise ValueError('gated_act: needs an even number of columns (a multiple of 32 when they are interleaved)')
+    pointer, code, splits = _operand(gate_up, 'gate_up', out_dtype, (n, both))
+    out = torch.empty((n, both // 2), dtype=out_dtype, device=gate_up.device)
+    _check(library.load().qil_gated_act(pointer, code, splits, _ptr(out), n, both // 2, _code(out_dtype), int(interleaved),
+                                        GATE_FUNCTIONS[activation], float(limit), float(alpha), _stream()), 'gated_act')
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Attention over a cached latent
+def latent_prepare(down, *, q_rank, rank, rot, q_weight, c_weight, eps, frequencies, positions, slots, latent, rope,
+                   dtype):
+    """From the stacked down products ``down`` [N, q_rank + rank + rot] (tensor of ``dtype`` or Partials): the
+    RMS-normed query latent [N, q_rank] (returned); the RMS-normed key/value latent and the rotated shared key part go
+    into the caches ``latent`` [.., rank] / ``rope`` [.., rot] at ``slots`` (None: nothing is stored)."""
+    n = down.shape[0]
+    pointer, code, splits = _operand(down, 'down', dtype, (n, q_rank + rank + rot))
+    _require(q_weight, 'q_weight', torch.float32, (q_rank,))
+    _require(c_weight, 'c_weight', torch.float32, (rank,))
+    _require(frequencies, 'frequencies', torch.float32, (rot // 2,))
+    _require(positions, 'positions', torch.int32, (n,))
+    if slots is not None:
+        _require(slots, 'slots', torch.int32, (n,))
+        _require(latent, 'latent', dtype)
+        _require(rope, 'rope', dtype)
+        if latent.shape[-1] != rank or rope.shape[-1] != rot or latent.shape[:-1] != rope.shape[:-1]:
+            raise ValueError('latent_prepare: caches must be [.., rank] and [.., rot] over the same slots')
+    out = torch.empty((n, q_rank), dtype=dtype, device=down.device)
+    _check(library.load().qil_latent_prepare(pointer, code, splits, _ptr(q_weight), _ptr(c_weight), _ptr(frequencies),
+                                             _ptr(positions), _ptr(slots), _ptr(out), _ptr(latent), _ptr(rope), n, q_rank,
+                                             rank, rot, float(eps), _code(dtype), _stream()), 'latent_prepare')
+    return out
+
+
+def head_product(x, weight, *, heads, out_dtype, out=None, out_columns=None):
+    """A product per head: x [N, heads * X] (head h's K inputs lead its X columns), weight [heads, K, O] (for every k
+    its O outputs side by side) -> [N, heads * O] of ``out_dtype``, or into the leading O of every head's
+    ``out_columns`` columns of ``out``."""
+    n = x.shape[0]
+    _require(x, 'x')
+    _require(weight, 'weight')
+    if weight.ndim != 3 or weight.shape[0] != heads or x.shape[1] % heads or x.shape[1] // heads < weight.shape[1]:
+        raise ValueError(f'head_product: x {tuple(x.shape)}, weight {tuple(weight.shape)}, {heads} heads')
+    k, o = weight.shape[1], weight.shape[2]
+    if out is None:
+        out_columns = o
+        out = torch.empty((n, heads * o), dtype=out_dtype, device=x.device)
+    _require(out, 'out', out_dtype, (n, heads * out_columns))
+    _check(library.load().qil_head_product(_ptr(x), _code(x.dtype), x.shape[1], x.shape[1] // heads, _ptr(weight),
+                                           _code(weight.dtype), _ptr(out), _code(out_dtype), heads * out_columns,
+                                           out_columns, n, heads, k, o, _stream()), 'head_product')
+    return out
+
+
+def latent_query(q, k_up, *, heads, dim, rot, rank, frequencies, positions):
+    """Queries in the latent's space.  ``q`` [N, heads * (dim + rot)] (a head's unrotated part first), ``k_up``
+    [heads, dim, rank] (the key expansion, a head's rows, as stored) -> float32 [N, heads, rank + rot]:
+    k_up_h^T q_h, then the head's rotated part turned by the row's position."""
+    n = q.shape[0]
+    _require(q, 'q', None, (n, heads * (dim + rot)))
+    _require(k_up, 'k_up', q.dtype, (heads, dim, rank))
+    _require(frequencies, 'frequencies', torch.float32, (rot // 2,))
+    _require(positions, 'positions', torch.int32, (n,))
+    out = torch.empty((n, heads * (rank + rot)), dtype=torch.float32, device=q.device)
+    head_product(q, k_up, heads=heads, out_dtype=torch.float32, out=out, out_columns=rank + rot)
+    _check(library.load().qil_rotate_tail(_ptr(q), _code(q.dtype), heads * (dim + rot), dim + rot, dim, _ptr(frequencies),
+                                          _ptr(positions), _ptr(out), heads * (rank + rot), rank + rot, rank, n, heads,
+                                          rot, _stream()), 'rotate_tail')
+    return out
+
+
+def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, positions, sink, scale, heads, rank, rot):
+    """Every row's attention over its request's cached latents: ``q`` float32 [N, heads * (rank + rot)] as
+    ``latent_query`` makes it; caches [pages, page_size, rank] and [pages, page_size, rot]; row n sees keys
+    j <= positions[n] of sequence row_seq[n] (a row of ``block_tables``).  ``sink`` float32 [heads] or None: a logit
+    per head that counts once in the softmax's denominator and has no value.  -> float32 [N, heads * rank], the
+    weighted sums of the latents."""
+    n = q.shape[0]
+    _require(q, 'q', torch.float32, (n, heads * (rank + rot)))
+    _require(latent, 'latent')
+    _require(rope, 'rope', latent.dtype)
+    if tuple(latent.shape[1:]) != (page_size, rank) or tuple(rope.shape[1:]) != (page_size, rot) or \
+            latent.shape[0] != rope.shape[0]:
+        raise ValueError('latent_attention: caches must be [pages, page_size, rank] and [pages, page_size, rot]')
+    _require(block_tables, 'block_tables', torch.int32)
+    _require(row_seq, 'row_seq', torch.int32, (n,))
+    _require(positions, 'positions', torch.int32, (n,))
+    if sink is not None:
+        _require(sink, 'sink', torch.float32, (heads,))
+    lib = library.load()
+    if not lib.qil_latent_attention_takes(heads, rank, rot):
+        raise UnsupportedShape(f'latent attention: {heads} heads, rank {rank}, {rot} rotated elements')
+    out = torch.empty((n, heads * rank), dtype=torch.float32, device=q.device)
+    _check(lib.qil_latent_attention(_ptr(q), _ptr(latent), _ptr(rope), _ptr(block_tables), block_tables.shape[1],
+                                    _ptr(row_seq), _ptr(positions), _ptr(sink), _ptr(out), n, heads, rank, rot, page_size,
+                                    float(scale), _code(latent.dtype), _stream()), 'latent_attention')
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Recurrences with a matrix state
+SCAN_MODES = {'decay': 0, 'mlstm': 1}
+
+
+def state_scan_slot(*, heads, dim, vdim, mode):
+    """float32 elements of one request's state for ``state_scan``: the heads' [dim, vdim] matrices, and for 'mlstm' a
+    normaliser [dim] and a maximum per head and tile of 64 state columns (the kernel's blocks keep one each)."""
+    tiles = -(-vdim // 64)
+    return heads * dim * vdim + (heads * tiles * (dim + 1) if SCAN_MODES[mode] == SCAN_MODES['mlstm'] else 0)
+
+
+def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, state, cu_seqlens, seq_starts, seq_slots,
+               n_seqs, gates=None, gate_bias=None, cap=0.0, decay=None, frequencies=None, rot=0, q_scale=1.0, k_scale=1.0):
+    """S_t = a_t S_(t-1) + b_t k_t v_t^T, o_t = S_t^T q_t per head over every sequence's rows of the step, from the
+    sequence's state slot (empty where the sequence starts at position 0) and back into it.
+
+    ``proj`` [N, P]: a row holds the heads' queries from column ``q_offset``, keys from ``k_offset`` (heads * dim each)
+    and values from ``v_offset`` (heads * vdim).  Mode 'decay': a_t = decay[h], b_t = 1.  Mode 'mlstm': exponential
+    gates from ``gates`` float32 [N, 2 heads] (+ ``gate_bias`` [2 heads]; input gates first) soft-capped at ``cap``,
+    with a running maximum and a normaliser.  Queries and keys are rotated by position on their leading ``rot``
+    elements (``frequencies`` [rot / 2]) and then scaled.  -> float32 [N, heads * vdim]."""
+    n = proj.shape[0]
+    _require(proj, 'proj')
+    code = _code(proj.dtype)
+    lib = library.load()
+    if not lib.qil_state_scan_takes(dim, vdim, rot):
+        raise UnsupportedShape(f'state_scan: dim {dim} (up to 256), vdim {vdim}, {rot} rotated elements')
+    width = proj.shape[1]
+    if min(q_offset, k_offset, v_offset) < 0 or max(q_offset, k_offset) + heads * dim > width or v_offset + heads * vdim > width:
+        raise ValueError('state_scan: offsets do not fit the rows')
+    slot = state_scan_slot(heads=heads, dim=dim, vdim=vdim, mode=mode)
+    if slot != lib.qil_state_scan_slot(heads, dim, vdim, SCAN_MODES[mode]):
+        raise RuntimeError('state_scan: the kernel library lays a state slot out differently')
+    _require(state, 'state', torch.float32)
+    if state.ndim != 2 or state.shape[1] != slot:
+        raise ValueError(f'state_scan: state must be [slots, {slot}]')
+    _require(cu_seqlens, 'cu_seqlens', torch.int32, (n_seqs + 1,))
+    _require(seq_starts, 'seq_starts', torch.int32, (n_seqs,))
+    _require(seq_slots, 'seq_slots', torch.int32, (n_seqs,))
+    if mode == 'mlstm':
+        _require(gates, 'gates', torch.float32, (n, 2 * heads))
+        _require(gate_bias, 'gate_bias', torch.float32, (2 * heads,))
+    else:
+        _require(decay, 'decay', torch.float32, (heads,))
+    if rot:
+        _require(frequencies, 'frequencies', torch.float32, (rot // 2,))
+    out = torch.empty((n, heads * vdim), dtype=torch.float32, device=proj.device)
+    _check(lib.qil_state_scan(_ptr(proj), code, width, q_offset, k_offset, v_offset, _ptr(gates), _ptr(gate_bias),
+                              float(cap), _ptr(decay), _ptr(frequencies) if rot else None, rot, float(q_scale),
+                              float(k_scale), _ptr(state), _ptr(cu_seqlens), _ptr(seq_starts), _ptr(seq_slots), _ptr(out),
+                              n_seqs, heads, dim, vdim, SCAN_MODES[mode], _stream()), 'state_scan')
+    return out
+
+
+def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gate, out_dtype):
+    """Per head: o / sqrt(mean(o^2) + eps) (* weight) * act(g), ``o`` float32 [N, heads * vdim], g the heads * vdim
+    columns of ``gate_source`` from ``gate_offset``; ``gate``: 'sigmoid' or 'silu'.  -> [N, heads * vdim] out_dtype."""
+    n = o.shape[0]
+    _require(o, 'o', torch.float32, (n, heads * vdim))
+    _require(gate_source, 'gate_source', out_dtype)
+    if gate_source.shape[0] != n or gate_offset + heads * vdim > gate_source.shape[1]:
+        raise ValueError('head_norm_gate: the gate columns do not fit')
+    if weight is not None:
+        _require(weight, 'weight', torch.float32, (heads * vdim,))
+    out = torch.empty((n, heads * vdim), dtype=out_dtype, device=o.device)
+    _check(library.load().qil_head_norm_gate(_ptr(o), _ptr(gate_source), gate_source.shape[1], gate_offset, _ptr(weight),
+                                             _ptr(out), n, heads, vdim, float(eps), {'sigmoid': 0, 'silu': 1}[gate],
+                                             _code(out_dtype), _stream()), 'head_norm_gate')
+    return out

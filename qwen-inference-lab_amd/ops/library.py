@@ -287,6 +287,23 @@ def _declare(lib):
     lib.qil_gemm_bf16_wide_gated_takes.argtypes = [i, i, i]
     lib.qil_gemm_bf16_wide_gated_takes.restype = i
     lib.qil_gemm_bf16_wide_gated.argtypes = [p, p, p, i, i, i, i, p]
+    lib.qil_add_norm.argtypes = [p, p, i, i, i, f, p, p, p, i, i, f, i, i, i, p]
+    lib.qil_gated_act.argtypes = [p, i, i, p, i, i, i, i, i, f, f, p]
+    lib.qil_latent_prepare.argtypes = [p, i, i, p, p, p, p, p, p, p, p, i, i, i, i, f, i, p]
+    lib.qil_head_product.argtypes = [p, i, i, i, p, i, p, i, i, i, i, i, i, i, p]
+    lib.qil_rotate_tail.argtypes = [p, i, i, i, i, p, p, p, i, i, i, i, i, i, p]
+    lib.qil_latent_attention_takes.argtypes = [i, i, i]
+    lib.qil_latent_attention_takes.restype = i
+    lib.qil_latent_attention.argtypes = [p, p, p, p, i, p, p, p, p, i, i, i, i, i, f, i, p]
+    lib.qil_state_scan_slot.argtypes = [i, i, i, i]
+    lib.qil_state_scan_slot.restype = z
+    lib.qil_state_scan_takes.argtypes = [i, i, i]
+    lib.qil_state_scan_takes.restype = i
+    lib.qil_state_scan.argtypes = [p, i, i, i, i, i, p, p, f, p, p, i, f, f, p, p, p, p, p, i, i, i, i, i, p]
+    lib.qil_head_norm_gate.argtypes = [p, p, i, i, p, p, i, i, i, f, i, i, p]
+    for name in ('qil_add_norm', 'qil_gated_act', 'qil_latent_prepare', 'qil_head_product', 'qil_rotate_tail',
+                 'qil_latent_attention', 'qil_state_scan', 'qil_head_norm_gate'):
+        getattr(lib, name).restype = i
     lib.qil_sample.argtypes = [p, p, p, p, p, p, p, i, i, p]
     lib.qil_sample_workspace.argtypes = [i, i]
     lib.qil_sample_workspace.restype = z

@@ -1,14 +1,17 @@
 """Parts that models are assembled from."""
 from .base import (ParamSpec, KVNeed, PagedNeed, StateNeed, Part, Norm, PositionEncoding, Rotation,
                    Mixer, FeedForward, Block)
-from .norm import RMSNorm
-from .rotary import Rotary
+from .norm import RMSNorm, LayerNorm
+from .rotary import Rotary, RotaryFrequencies
 from .attention import Attention
+from .latent_attention import LatentAttention
+from .recurrent import MatrixMemory
 from .mlp import GatedMLP
 from .block import PreNormBlock
 from .embedding import Embedding, LMHead
 from .model import CausalLM, ScheduleEntry
 
 __all__ = ['ParamSpec', 'KVNeed', 'PagedNeed', 'StateNeed', 'Part', 'Norm', 'PositionEncoding', 'Rotation', 'Mixer',
-           'FeedForward', 'Block', 'RMSNorm', 'Rotary', 'Attention', 'GatedMLP', 'PreNormBlock',
+           'FeedForward', 'Block', 'RMSNorm', 'LayerNorm', 'Rotary', 'RotaryFrequencies', 'Attention',
+           'LatentAttention', 'MatrixMemory', 'GatedMLP', 'PreNormBlock',
            'Embedding', 'LMHead', 'CausalLM', 'ScheduleEntry']

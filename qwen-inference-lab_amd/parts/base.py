@@ -79,6 +79,8 @@ class Norm(Part):
     into ``stream`` in place (float32 sum), then the sum is normalised.
     ``forward_rows(stream, delta, rows, out_dtype)``: the same for the selected
     rows only, leaving ``stream`` untouched.
+    A block whose residual sums are scaled (x + m * sublayer(x)) passes ``delta_scale=m`` to both; blocks that do not
+    scale never pass it.
     """
     def forward(self, stream, delta, out_dtype):
         raise NotImplementedError

@@ -6,16 +6,19 @@ from .. import ops
 
 
 class GatedMLP(FeedForward):
-    """``activation`` names the gate's function; 'silu' (z * sigmoid(z)) is the one
-    the kernels have.  Gate and up matrices become one [2 * intermediate, width] matrix at
+    """``activation`` names the gate's function (``ops.GATE_FUNCTIONS``): 'silu', silu(g) * u, or 'clamped_swish' with
+    ``limit`` L and ``alpha`` a: g' = min(g, L), u' = clamp(u, -L, L), g' * sigmoid(a g') * (u' + 1).  Gate and up matrices become one [2 * intermediate, width] matrix at
     ``finalize`` (rows in turns of 16, or gate rows first where the sizes do not allow that): a pure re-layout."""
 
-    def __init__(self, *, width, intermediate, activation='silu', dtype=torch.bfloat16):
+    def __init__(self, *, width, intermediate, activation='silu', limit=None, alpha=1.0, dtype=torch.bfloat16):
         super().__init__()
         self.dtype = dtype
-        if activation != 'silu':
+        if activation not in ops.GATE_FUNCTIONS:
             raise ValueError(f'no kernel for activation {activation!r}')
+        if activation == 'clamped_swish' and not (limit is not None and limit > 0):
+            raise ValueError('clamped_swish needs a positive limit')
         self.width, self.intermediate, self.activation = width, intermediate, activation
+        self.limit, self.alpha = float(limit or 0.0), float(alpha)
 
     def param_specs(self):
         return {'gate_proj.weight': ParamSpec((self.intermediate, self.width)),
@@ -32,7 +35,8 @@ class GatedMLP(FeedForward):
     adds_to_stream = True
 
     def forward(self, h, add_to=None):
-        hidden = ops.gated_linear(h, self.p['gate_up_proj.weight'], self.dtype, interleaved=self.interleaved, lazy=True)
+        hidden = ops.gated_linear(h, self.p['gate_up_proj.weight'], self.dtype, interleaved=self.interleaved, lazy=True,
+                                  activation=self.activation, limit=self.limit, alpha=self.alpha)
         if add_to is not None and hidden.is_cuda:              # few rows: the down product adds into the stream itself
             return ops.linear(hidden, self.p['down_proj.weight'], None, partials=True, add_to=add_to)
         return ops.linear(hidden, self.p['down_proj.weight'], None, partials=True)

@@ -30,7 +30,9 @@ class CausalLM:
     """
 
     def __init__(self, *, config, embedding, blocks, schedule, final_norm, head, names, tied=None,
-                 dtype=torch.bfloat16, device='cuda'):
+                 dtype=torch.bfloat16, device='cuda', residual_scale=1.0):
+        self.residual_scale = float(residual_scale)     # what the last block's output is multiplied by as it is added
+        self.observer = None                            # callable(schedule position, stream, pending, scale) or None
         self.config, self.embedding, self.blocks, self.schedule = config, embedding, list(blocks), list(schedule)
         self.final_norm, self.head, self.names, self.tied = final_norm, head, dict(names), dict(tied or {})
         self.dtype, self.device = dtype, torch.device(device)
@@ -98,11 +100,17 @@ class CausalLM:
         """
         stream = self.embedding.forward_step(ctx)
         pending = None
-        for entry, cache in zip(self.schedule, caches):
+        for position, (entry, cache) in enumerate(zip(self.schedule, caches)):
             pending = self.blocks[entry.block].forward(stream, pending, ctx, cache)
+            if self.observer is not None:                       # the stream after this run is stream + scale * pending
+                self.observer(position, stream, pending, self.residual_scale)
         if ctx.n_logit_rows == 0:
             return None
         if isinstance(pending, ops.Added):                      # the last block's output is in the stream already
             pending = None
-        rows = self.final_norm.forward_rows(stream, pending, ctx.logit_rows, self.dtype)
+        if self.residual_scale != 1.0:
+            rows = self.final_norm.forward_rows(stream, pending, ctx.logit_rows, self.dtype,
+                                                delta_scale=self.residual_scale)
+        else:
+            rows = self.final_norm.forward_rows(stream, pending, ctx.logit_rows, self.dtype)
         return self.head.forward(rows)

@@ -1,4 +1,4 @@
-"""RMSNorm with float32 statistics.  Formula: qil/model.py:15-23."""
+"""Norms with float32 statistics: RMSNorm (formula: qil/model.py:15-23) and a layer norm without a bias."""
 import torch
 
 from .base import Norm, ParamSpec
@@ -15,7 +15,9 @@ class RMSNorm(Norm):
     def param_specs(self):
         return {'weight': ParamSpec((self.width,), 'vector', 'one_plus_normal')}
 
-    def forward(self, stream, delta, out_dtype):
+    def forward(self, stream, delta, out_dtype, delta_scale=1.0):
+        if delta_scale != 1.0:                      # (the general kernel rounds once, after the weight)
+            return ops.add_norm(stream, delta, self.p['weight'], self.eps, out_dtype, centre=False, delta_scale=delta_scale)
         return ops.add_rmsnorm(stream, delta, self.p['weight'], self.eps, out_dtype)
 
     def forward_lazy(self, stream, out_dtype, added):
@@ -23,5 +25,27 @@ class RMSNorm(Norm):
             return ops.Normed(stream, self.p['weight'], self.eps, out_dtype, added)
         return None
 
-    def forward_rows(self, stream, delta, rows, out_dtype):
+    def forward_rows(self, stream, delta, rows, out_dtype, delta_scale=1.0):
+        if delta_scale != 1.0:
+            return ops.rows_norm(stream, delta, rows, self.p['weight'], self.eps, out_dtype, centre=False,
+                                 delta_scale=delta_scale)
         return ops.rows_rmsnorm(stream, delta, rows, self.p['weight'], self.eps, out_dtype)
+
+
+class LayerNorm(Norm):
+    """y = (x - mean(x)) / sqrt(mean((x - mean(x))^2) + eps) * weight: a weight, no bias; float32 throughout and one
+    rounding of the result.  ``delta_scale`` multiplies the sub-layer output that is added into the stream first."""
+
+    def __init__(self, width, eps):
+        super().__init__()
+        self.width, self.eps = int(width), float(eps)
+
+    def param_specs(self):
+        return {'weight': ParamSpec((self.width,), 'vector', 'one_plus_normal')}
+
+    def forward(self, stream, delta, out_dtype, delta_scale=1.0):
+        return ops.add_norm(stream, delta, self.p['weight'], self.eps, out_dtype, centre=True, delta_scale=delta_scale)
+
+    def forward_rows(self, stream, delta, rows, out_dtype, delta_scale=1.0):
+        return ops.rows_norm(stream, delta, rows, self.p['weight'], self.eps, out_dtype, centre=True,
+                             delta_scale=delta_scale)

@@ -33,3 +33,24 @@ class Rotary(PositionEncoding):
             self._rotation = Rotation(angles.cos().to(self.device).contiguous(),
                                       angles.sin().to(self.device).contiguous(), self.rot_dim)
         return self._rotation
+
+
+class RotaryFrequencies(PositionEncoding):
+    """The rotation as its frequencies alone: f_i = base**(-2 i / rot_dim), i < rot_dim / 2, made in float64 and held
+    in float32.  Kernels that take it make the angle position * f_i and its cosine and sine themselves, in float32,
+    so no table bounds the positions.  Pairing is (i, i + rot_dim / 2)."""
+
+    def __init__(self, rot_dim, base, *, device='cpu'):
+        super().__init__()
+        self.rot_dim, self.base, self.device = int(rot_dim), float(base), device
+        if self.rot_dim < 2 or self.rot_dim % 2:
+            raise ValueError('rot_dim must be even and at least 2')
+        if not self.base > 0:
+            raise ValueError('the base must be positive')
+        self._frequencies = None
+
+    def frequencies(self):
+        if self._frequencies is None:
+            values = [self.base ** (-2.0 * i / self.rot_dim) for i in range(self.rot_dim // 2)]
+            self._frequencies = torch.tensor(values, dtype=torch.float64).to(torch.float32).to(self.device).contiguous()
+        return self._frequencies

@@ -1,8 +1,8 @@
 """The one registry: architecture name -> (configuration class, model builder).
 
-``config.json["architectures"][0]`` selects the entry everywhere in the engine
-(loader, random-weights writer, command line, trace replay).  A folder without
-``architectures`` is matched by its ``model_type``.  The reference has a single
+``config.json["architectures"][0]`` (or a single name under ``"architecture"``) selects the entry
+everywhere in the engine (loader, random-weights writer, command line, trace replay).  A folder with
+neither is matched by its ``model_type``.  The reference has a single
 hard-wired check instead (qil/config.py:37, qil/__main__.py:25,33).
 
 An entry's ``build(config, dtype=, device=)`` returns an unloaded model
@@ -41,6 +41,8 @@ def architecture_for(data):
     """Entry for a parsed config.json dict."""
     _load_builtin()
     names = data.get('architectures')
+    if not names and isinstance(data.get('architecture'), str):
+        names = [data['architecture']]
     if names:
         if not isinstance(names, list) or not isinstance(names[0], str):
             raise ConfigError("'architectures' must be a list of names")

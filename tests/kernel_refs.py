@@ -55,10 +55,17 @@ def _halves(gate_up, interleaved):
     return tiles[:, :, 0].reshape(-1, inner), tiles[:, :, 1].reshape(-1, inner)
 
 
-def gated_linear(x, weight, out_dtype=None, interleaved=False, lazy=False):
+def _gate(g, u, activation='silu', limit=0.0, alpha=1.0):
+    if activation == 'clamped_swish':
+        g, u = g.clamp(max=limit), u.clamp(min=-limit, max=limit)
+        return g / (1 + torch.exp(-alpha * g)) * (u + 1)
+    return g / (1 + torch.exp(-g)) * u
+
+
+def gated_linear(x, weight, out_dtype=None, interleaved=False, lazy=False, activation='silu', limit=0.0, alpha=1.0):
     y = x.to(torch.float32) @ weight.to(torch.float32).t()
     g, u = _halves(y, interleaved)
-    return (g / (1 + torch.exp(-g)) * u).to(out_dtype or x.dtype)
+    return _gate(g, u, activation, limit, alpha).to(out_dtype or x.dtype)
 
 
 def silu_mul(gate_up, out_dtype=None, interleaved=False):
