@@ -155,5 +155,148 @@ def sample(logits, temperatures, seeds, counters, out=None):
     return tokens, finite
 
 
+def _any_norm(x, weight, eps, centre):
+    if centre:
+        x = x - x.mean(dim=-1, keepdim=True)
+    return x / torch.sqrt(x.square().mean(dim=-1, keepdim=True) + eps) * weight
+
+
+def add_norm(stream, delta, weight, eps, out_dtype, *, centre, delta_scale=1.0):
+    if delta is not None:
+        stream += delta_scale * _value(delta).to(torch.float32)
+    return _any_norm(stream, weight, eps, centre).to(out_dtype)
+
+
+def rows_norm(stream, delta, rows, weight, eps, out_dtype, *, centre, delta_scale=1.0):
+    x = stream[rows.long()]
+    if delta is not None:
+        x = x + delta_scale * _value(delta)[rows.long()].to(torch.float32)
+    return _any_norm(x, weight, eps, centre).to(out_dtype)
+
+
+def gated_act(gate_up, out_dtype, *, activation, limit=0.0, alpha=1.0, interleaved=False):
+    g, u = (t.to(torch.float32) for t in _halves(_value(gate_up), interleaved))
+    return _gate(g, u, activation, limit, alpha).to(out_dtype)
+
+
+def _turn(x, positions, frequencies):
+    """x [N, ..., rot]: element i with i + rot / 2, angle position * frequencies[i]; float32."""
+    half = x.shape[-1] // 2
+    angle = positions.to(torch.float32)[:, None] * frequencies[None, :]
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [half]
+    cos, sin = angle.cos().reshape(shape), angle.sin().reshape(shape)
+    u, v = x[..., :half], x[..., half:]
+    return torch.cat([u * cos - v * sin, v * cos + u * sin], dim=-1)
+
+
+def latent_prepare(down, *, q_rank, rank, rot, q_weight, c_weight, eps, frequencies, positions, slots, latent, rope,
+                   dtype):
+    x = _value(down).to(torch.float32)
+    cq = _any_norm(x[:, :q_rank], q_weight, eps, False).to(dtype)
+    if slots is not None:
+        latent.view(-1, rank)[slots.long()] = _any_norm(x[:, q_rank:q_rank + rank], c_weight, eps, False).to(dtype)
+        rope.view(-1, rot)[slots.long()] = _turn(x[:, q_rank + rank:], positions, frequencies).to(dtype)
+    return cq
+
+
+def head_product(x, weight, *, heads, out_dtype, out=None, out_columns=None):
+    n, k, o = x.shape[0], weight.shape[1], weight.shape[2]
+    result = torch.einsum('nhk,hko->nho', x.to(torch.float32).view(n, heads, -1)[:, :, :k], weight.to(torch.float32))
+    if out is None:
+        return result.reshape(n, heads * o).to(out_dtype)
+    out.view(n, heads, out_columns)[:, :, :o] = result.to(out_dtype)
+    return out
+
+
+def latent_query(q, k_up, *, heads, dim, rot, rank, frequencies, positions):
+    n = q.shape[0]
+    q = q.to(torch.float32).view(n, heads, dim + rot)
+    absorbed = torch.einsum('nhd,hdr->nhr', q[:, :, :dim], k_up.to(torch.float32))
+    return torch.cat([absorbed, _turn(q[:, :, dim:], positions, frequencies)], dim=-1).reshape(n, heads * (rank + rot))
+
+
+def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, positions, sink, scale, heads, rank, rot):
+    n = q.shape[0]
+    q = q.view(n, heads, rank + rot)
+    out = torch.zeros((n, heads, rank), dtype=torch.float32)
+    flat_c, flat_r = latent.view(-1, rank).to(torch.float32), rope.view(-1, rot).to(torch.float32)
+    for row in range(n):
+        keys = torch.arange(int(positions[row]) + 1)
+        table = block_tables[int(row_seq[row])].long()
+        slots = table[keys // page_size] * page_size + keys % page_size
+        c, r = flat_c[slots], flat_r[slots]
+        scores = (q[row, :, :rank] @ c.t() + q[row, :, rank:] @ r.t()) * scale                  # [heads, keys]
+        if sink is not None:
+            scores = torch.cat([scores, sink[:, None]], dim=1)
+        p = torch.softmax(scores, dim=1)[:, :len(keys)]
+        out[row] = p @ c
+    return out.reshape(n, heads * rank)
+
+
+def state_scan_slot(*, heads, dim, vdim, mode):
+    tiles = -(-vdim // 64)
+    return heads * dim * vdim + (heads * tiles * (dim + 1) if mode == 'mlstm' else 0)
+
+
+def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, state, cu_seqlens, seq_starts, seq_slots,
+               n_seqs, gates=None, gate_bias=None, cap=0.0, decay=None, frequencies=None, rot=0, q_scale=1.0, k_scale=1.0):
+    """The state slot's layout is the kernel's: matrices, then per head and tile of 64 columns a normaliser and a maximum."""
+    n, tiles = proj.shape[0], -(-vdim // 64)
+    x = proj.to(torch.float32)
+    q = x[:, q_offset:q_offset + heads * dim].reshape(n, heads, dim).clone()
+    k = x[:, k_offset:k_offset + heads * dim].reshape(n, heads, dim).clone()
+    v = x[:, v_offset:v_offset + heads * vdim].reshape(n, heads, vdim)
+    out = torch.zeros((n, heads, vdim), dtype=torch.float32)
+    mats = heads * dim * vdim
+    for s in range(n_seqs):
+        lo, hi, start, slot = int(cu_seqlens[s]), int(cu_seqlens[s + 1]), int(seq_starts[s]), int(seq_slots[s])
+        positions = torch.arange(start, start + hi - lo)
+        qs, ks = q[lo:hi], k[lo:hi]
+        if rot:
+            qs = torch.cat([_turn(qs[..., :rot], positions, frequencies), qs[..., rot:]], dim=-1)
+            ks = torch.cat([_turn(ks[..., :rot], positions, frequencies), ks[..., rot:]], dim=-1)
+        qs, ks = qs * q_scale, ks * k_scale
+        fresh = start == 0
+        memory = torch.zeros(heads, dim, vdim) if fresh else state[slot, :mats].view(heads, dim, vdim).clone()
+        if mode == 'mlstm':
+            norms = state[slot, mats:mats + heads * tiles * dim].view(heads, tiles, dim)
+            tops = state[slot, mats + heads * tiles * dim:].view(heads, tiles)
+            norm = torch.zeros(heads, dim) if fresh else norms[:, 0].clone()
+            top = torch.zeros(heads) if fresh else tops[:, 0].clone()
+        for t in range(hi - lo):
+            if mode == 'mlstm':
+                pre = gates[lo + t] + gate_bias
+                log_in = cap * torch.tanh(pre[:heads] / cap)
+                log_keep = torch.nn.functional.logsigmoid(cap * torch.tanh(pre[heads:] / cap))
+                now = torch.maximum(log_keep + top, log_in)
+                a, b, top = torch.exp(log_keep + top - now), torch.exp(log_in - now), now
+            else:
+                a, b = decay, torch.ones(heads)
+            memory = a[:, None, None] * memory + b[:, None, None] * ks[t][:, :, None] * v[lo + t][:, None, :]
+            read = torch.einsum('hdv,hd->hv', memory, qs[t])
+            if mode == 'mlstm':
+                norm = a[:, None] * norm + b[:, None] * ks[t]
+                read = read / (torch.maximum((norm * qs[t]).sum(-1).abs(), torch.exp(-top)) + 1e-6)[:, None]
+            out[lo + t] = read
+        state[slot, :mats] = memory.reshape(-1)
+        if mode == 'mlstm':
+            norms[:] = norm[:, None, :]
+            tops[:] = top[:, None]
+    return out.reshape(n, heads * vdim)
+
+
+def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gate, out_dtype):
+    n = o.shape[0]
+    unit = o.view(n, heads, vdim)
+    unit = (unit / torch.sqrt(unit.square().mean(dim=-1, keepdim=True) + eps)).reshape(n, heads * vdim)
+    if weight is not None:
+        unit = unit * weight
+    g = gate_source[:, gate_offset:gate_offset + heads * vdim].to(torch.float32)
+    return (unit * (torch.sigmoid(g) if gate == 'sigmoid' else g * torch.sigmoid(g))).to(out_dtype)
+
+
 ALL = dict(embed=embed, add_rmsnorm=add_rmsnorm, rows_rmsnorm=rows_rmsnorm, linear=linear, gated_linear=gated_linear, silu_mul=silu_mul,
-           qk_norm_rope_store=qk_norm_rope_store, paged_attention=paged_attention, sample=sample)
+           qk_norm_rope_store=qk_norm_rope_store, paged_attention=paged_attention, sample=sample,
+           add_norm=add_norm, rows_norm=rows_norm, gated_act=gated_act, latent_prepare=latent_prepare, head_product=head_product,
+           latent_query=latent_query, latent_attention=latent_attention, state_scan_slot=state_scan_slot, state_scan=state_scan,
+           head_norm_gate=head_norm_gate)
