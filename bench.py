@@ -193,6 +193,95 @@ def attention_phase(args, torch, config, dtype):
     return 0
 
 
+
+# ---------------------------------------------------------------------------------------------------------------
+# --phase designs: the Fubapel design beside dense Qwen3 at equal sizes (width, feed-forward, layers, heads x head size)
+DESIGN_SIZES = {
+    # width, feed-forward, heads, head size of the attention; the latent's ranks; the memories' heads and head sizes
+    '1b': dict(width=2048, ff=6144, heads=16, dim=128, rot_dim=64, kv_rank=512, q_rank=1536, memory_heads=8, memory_dim=128,
+               memory_vdim=256),
+    '8b': dict(width=4096, ff=12288, heads=32, dim=128, rot_dim=64, kv_rank=512, q_rank=1536, memory_heads=16, memory_dim=128,
+               memory_vdim=256),
+}
+
+
+def fubapel_config(z, layers, vocab):
+    """`layers` layers in turns of latent attention, gated memory, decaying memory; a feed-forward behind each."""
+    ffn = dict(kind='dense', ff=z['ff'], limit=7.0)
+    kinds = [
+        dict(type='latent_attention', mlp=ffn,
+             mixer=dict(heads=z['heads'], dim=z['dim'], rot_dim=z['rot_dim'], vdim=z['dim'], kv_rank=z['kv_rank'],
+                        q_rank=z['q_rank'], rot=dict(base=10000.0, dims=z['rot_dim']), scale=(z['dim'] + z['rot_dim']) ** -0.5)),
+        dict(type='mlstm', mlp=ffn, mixer=dict(heads=z['memory_heads'], dim=z['memory_dim'], vdim=z['memory_vdim'], gate_cap=15.0)),
+        dict(type='retention', mlp=ffn,
+             mixer=dict(heads=z['memory_heads'], dim=z['memory_dim'], vdim=z['memory_vdim'],
+                        decay=[1 - 2.0 ** (-5 - i % 8) for i in range(z['memory_heads'])],
+                        rot=dict(base=10000.0, dims=z['memory_dim']))),
+    ]
+    return dict(architecture='Fubapel', vocab=vocab, width=z['width'], layers=[kinds[i % 3] for i in range(layers)],
+                loop=dict(start=0, stop=0, times=1), norm=dict(eps=1e-5), residual_mult=1.0)
+
+
+def designs_phase(args, torch, dtype):
+    """Prefill tokens a second and decode milliseconds a step of Fubapel models whose layers are all of one kind (and of
+    the three kinds in turns), beside dense Qwen3 of the same width, feed-forward, depth and attention heads."""
+    from qil_amd import Engine, Qwen3
+    from qil_amd.engine import ModelRunner, StepEntry
+    z, layers, vocab, page_size = DESIGN_SIZES[args.design_sizes], args.layers or 6, 32768, 16
+    generator = torch.Generator().manual_seed(99)
+    mixed = fubapel_config(z, layers, vocab)
+    models = {'fubapel (kinds in turns)': mixed}
+    for index, name in enumerate(('latent attention', 'gated memory', 'decaying memory')):
+        models[f'fubapel ({name} only)'] = dict(mixed, layers=[mixed['layers'][index]] * layers)
+    models['qwen3 (equal sizes)'] = dict(SIZES, vocab_size=vocab, hidden_size=z['width'], intermediate_size=z['ff'],
+                                         num_hidden_layers=layers, num_attention_heads=z['heads'],
+                                         num_key_value_heads=max(1, z['heads'] // 4), head_dim=z['dim'],
+                                         max_position_embeddings=max(args.history + args.steps + args.warmup + 64, args.prefill_tokens))
+    report = {'phase': 'designs', 'sizes': args.design_sizes, 'layers': layers, 'dtype': args.dtype,
+              'prefill_tokens': args.prefill_tokens, 'batch': args.batch, 'history': args.history, 'models': {}}
+    for name, config in models.items():
+        model = Qwen3.from_config(config, seed=0, dtype=dtype, device='cuda:0', on_device=True)
+        tokens = lambda n: torch.randint(0, vocab, (n,), generator=generator).tolist()
+        runner = ModelRunner(model, num_pages=-(-args.prefill_tokens // page_size) + 1, page_size=page_size, max_requests=1)
+        times = []
+        for attempt in range(4):
+            runner.admit(attempt)
+            ids = tuple(tokens(args.prefill_tokens))
+            torch.cuda.synchronize()
+            started = time.perf_counter()
+            logits = runner.step([StepEntry(attempt, ids, (args.prefill_tokens - 1,))])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - started)
+            assert torch.isfinite(logits).all()
+            runner.release(attempt)
+        prefill_s = statistics.median(times[1:])
+        del runner
+        new_tokens = args.warmup + args.steps + 8
+        pages = args.batch * (-(-(args.history + new_tokens) // page_size) + 1)
+        engine = Engine(model, num_pages=pages, page_size=page_size, token_budget=args.history + args.batch,
+                        prefill_chunk=args.history, max_active=args.batch)
+        ids = [engine.submit(tokens(args.history), max_new_tokens=new_tokens, ignore_eos=True) for _ in range(args.batch)]
+        while any(engine.result(i)['state'] == 'waiting' or engine.scheduler.computed(i) < args.history for i in ids):
+            engine.step()
+        for _ in range(args.warmup):
+            engine.step()
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        for _ in range(args.steps):
+            assert len(engine.step()) == args.batch
+        torch.cuda.synchronize()
+        step_s = (time.perf_counter() - started) / args.steps
+        engine.close()
+        report['models'][name] = {'prefill_ms': round(prefill_s * 1e3, 3), 'prefill_tokens_per_s': round(args.prefill_tokens / prefill_s, 1),
+                                  'decode_ms_per_step': round(step_s * 1e3, 4), 'decode_tokens_per_s': round(args.batch / step_s, 1),
+                                  'parameter_mb': round(model.parameter_bytes() / 1e6, 1)}
+        print(f'[bench] {name}: prefill {prefill_s * 1e3:.2f} ms, decode {step_s * 1e3:.3f} ms/step', file=sys.stderr, flush=True)
+        del engine, model
+        torch.cuda.empty_cache()
+    print(json.dumps(report))
+    return 0
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument('--gpus', type=int, default=1)
@@ -206,12 +295,14 @@ def main():
     parser.add_argument('--dtype', default='bfloat16', choices=['bfloat16', 'float32'])
     parser.add_argument('--points', default='1,64', help='other decode batch sizes to report, comma separated')
     parser.add_argument('--prefill-tokens', type=int, default=2048)
-    parser.add_argument('--phase', default='all', choices=['all', 'decode', 'prefill', 'e2e', 'mixed', 'attention', 'products'],
+    parser.add_argument('--phase', default='all', choices=['all', 'decode', 'prefill', 'e2e', 'mixed', 'attention', 'products', 'designs'],
                         help='measure only one phase (for profiling); the JSON line then lacks the other.  e2e: the '
                              'reference\'s own workloads (output tokens over the wall time of whole requests).  '
                              'mixed: steps of one prompt portion (--portion tokens) beside --batch decoded rows.  attention: the '
                              'attention kernels alone, at the reference\'s own shapes and at the benchmark\'s.  products: a layer\'s '
-                             'matrix products at --prefill-tokens rows alone, GPU BLAS against own kernel')
+                             'matrix products at --prefill-tokens rows alone, GPU BLAS against own kernel.  designs: prefill and decode of the '
+                             'Fubapel design at --design-sizes beside dense Qwen3 of equal sizes (--layers, default 6)')
+    parser.add_argument('--design-sizes', default='1b', choices=sorted(DESIGN_SIZES), help='layer sizes of --phase designs')
     parser.add_argument('--portion', type=int, default=128, help='tokens of the prompt portion of a mixed step')
     parser.add_argument('--own-products', action='store_true',
                         help='bfloat16 matrix products of many rows on this library\'s kernels instead of the GPU BLAS '
@@ -226,6 +317,8 @@ def main():
     from qil_amd import ops
     from qil_amd.engine import ModelRunner, StepEntry
     ops.OWN_LARGE_PRODUCTS = args.own_products
+    if args.phase == 'designs':
+        return designs_phase(args, torch, getattr(torch, args.dtype))
 
     sizes = dict(SIZES, **OTHER_SIZES[args.sizes])
     if args.layers is None:

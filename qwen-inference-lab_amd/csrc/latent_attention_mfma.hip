@@ -1,0 +1,310 @@
+// Attention over a cached latent on the matrix cores (bfloat16 caches): the arithmetic of latent_attention.hip,
+//     score(h, j) = scale * (qa_h . c_j + qr_h . kr_j),   u_h = sum_j p(h, j) c_j,   a sink logit in the denominator,
+// with v_mfma_f32_16x16x32_bf16.  Every head reads the same cached row [c_j ; kr_j], so a block stages a tile of 32
+// keys in LDS once and serves up to 64 query columns with it: a column is a (row, head) pair, the block's columns
+// are `rt` consecutive rows of one sequence times `hb` heads.  A wave owns 16 columns:
+//
+//   S^T[key, column] = sum_dim K[key, dim] Q[column, dim]       A = staged key rows, B = the wave's queries (registers)
+//   U^T[dim, column] = sum_key C^T[dim, key] P^T[key, column]    A = the tile's latents transposed, B = probabilities
+//
+// The value of a key is its own latent, so the same staged tile feeds both products; the second needs it with the
+// keys along a row, and the staging writes that transposed copy beside the plain one.  Row r of a 16-key score
+// sub-tile is key 8 (r / 4) + 4 jt + r % 4 of the 32-key step, so that a lane's eight scores are the eight consecutive
+// keys 8 kb .. 8 kb + 7 and go into the second product's B operand as they are.  Scores, maxima, exponentials, sums
+// and results are float32; probabilities enter the second product as bfloat16.
+//
+// With few blocks the keys go in parts (grid.z): a block leaves (maximum, sum, unnormalised result) per column and
+// part, and latent_merge_kernel finishes, which is also where the sink enters then.
+//
+// Takes rank % 16 == 0, rot % 8 == 0, rank + rot <= 640, rank <= 512; other sizes run on the general kernel.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define LM_THREADS 256
+#define LM_KEYS 32
+#define LM_VROW (LM_KEYS + 8)                               // elements of a row of the transposed tile (80 bytes)
+#define LOG2E 1.44269504088896f
+
+// EXACT: the sizes are the template's (rank + rot == 32 QF up to padding, rank == 16 VT): no size guards the products.
+template <int QF, int VT, bool EXACT>
+__global__ void __launch_bounds__(LM_THREADS)
+latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ latent, const bf16_t* __restrict__ rope,
+                   const int* __restrict__ tables, int table_stride, const int* __restrict__ cu_seqlens,
+                   const int* __restrict__ seq_starts, int n_seqs, int single, const float* __restrict__ sink,
+                   float* __restrict__ out, float* __restrict__ part_acc, float* __restrict__ part_m,
+                   float* __restrict__ part_l, int heads, int rank, int rot, int page_size, float scale, int rt, int hb,
+                   int P, int parts) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int d = rank + rot;
+  const int qf = EXACT ? QF : (d + 31) / 32, vt = EXACT ? VT : rank / 16;
+  const int dp = qf * 32, krow = dp + 8;
+  bf16_t* ks = reinterpret_cast<bf16_t*>(smem);            // [32 keys][krow]: c then kr then zeros
+  bf16_t* vts = ks + LM_KEYS * krow;                        // [rank][LM_VROW]: the latents, keys along a row
+
+  // which rows: tile `tile` of rt rows of sequence s
+  int s = 0, tile = blockIdx.x;
+  if (single) {
+    s = blockIdx.x;
+    tile = 0;
+  } else {
+    for (; s < n_seqs; ++s) {
+      const int tiles = (cu_seqlens[s + 1] - cu_seqlens[s] + rt - 1) / rt;
+      if (tile < tiles) break;
+      tile -= tiles;
+    }
+  }
+  if (s >= n_seqs) return;
+  const int seq_row0 = cu_seqlens[s], seq_rows = cu_seqlens[s + 1] - seq_row0, start = seq_starts[s];
+  const int r0 = tile * rt, rows_here = min(rt, seq_rows - r0);
+  const int last_pos = start + r0 + rows_here - 1;
+  const int h0 = blockIdx.y * hb, heads_here = min(hb, heads - h0);
+  const int part = blockIdx.z;
+  const int begin = part * P, end = min((part + 1) * P, last_pos + 1);
+  if (begin >= end) return;                                 // no row of the tile sees this part; the merge does not read it
+  const int* table = tables + (size_t)s * table_stride;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, kb = lane >> 4;
+  const int column = wave * 16 + r, ci = column / hb, ch = column - ci * hb;
+  const bool valid = ci < rows_here && ch < heads_here && column < rt * hb;
+  const bool working = wave * 16 < rt * hb;                 // wave-uniform: this wave has columns at all
+  const int grow = seq_row0 + r0 + (valid ? ci : 0), head = h0 + (valid ? ch : 0);
+  const int pos = valid ? start + r0 + ci : -1;
+  const size_t gcol = (size_t)grow * heads + head;
+
+  bf16x8 qb[QF];
+  {
+    const float* qrow = q + gcol * d;
+#pragma unroll
+    for (int f = 0; f < QF; ++f) {
+      float x[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int dim = 32 * f + 8 * kb + e;
+        x[e] = (valid && f < qf && dim < d) ? qrow[dim] : 0.f;
+      }
+      qb[f] = __builtin_bit_cast(bf16x8, make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]),
+                                                    pack_bf16(x[6], x[7])));
+    }
+  }
+  float m = -INFINITY, l = 0.f;
+  if (parts == 1 && sink && valid) {                       // the sink: maximum s_h, sum 1 (held once a column), result 0
+    m = sink[head];
+    l = kb == 0 ? 1.f : 0.f;
+  }
+  f32x4 o[VT];
+#pragma unroll
+  for (int t = 0; t < VT; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const int chunks = dp / 8;
+  for (int j0 = begin; j0 < end; j0 += LM_KEYS) {
+    __syncthreads();                                        // the last step's reads are done
+    for (int idx = tid; idx < LM_KEYS * chunks; idx += LM_THREADS) {
+      const int j = idx / chunks, dim = (idx - j * chunks) * 8, key = j0 + j;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (key < end && dim < d) {
+        const size_t slot = (size_t)table[key / page_size] * page_size + key % page_size;
+        v = dim < rank ? *reinterpret_cast<const uint4*>(latent + slot * rank + dim)
+                       : *reinterpret_cast<const uint4*>(rope + slot * rot + (dim - rank));
+      }
+      *reinterpret_cast<uint4*>(ks + j * krow + dim) = v;
+      if (dim < rank) {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          vts[(dim + 2 * e) * LM_VROW + j] = (bf16_t)(w[e] & 0xffffu);
+          vts[(dim + 2 * e + 1) * LM_VROW + j] = (bf16_t)(w[e] >> 16);
+        }
+      }
+    }
+    __syncthreads();
+    if (!working) continue;
+    // ---- scores
+    f32x4 sc[2];
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt) {
+      const bf16_t* krow_p = ks + (8 * (r >> 2) + 4 * jt + (r & 3)) * krow + 8 * kb;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int f = 0; f < QF; ++f)
+        if (EXACT || f < qf)
+          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(krow_p + 32 * f), qb[f], acc, 0, 0, 0);
+      sc[jt] = acc;
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = j0 + 8 * kb + 4 * jt + i;
+        const float v = (key <= pos && key < end) ? sc[jt][i] * scale : -INFINITY;
+        sc[jt][i] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, QIL_WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, QIL_WAVE));
+    const float m_new = fmaxf(m, mx);
+    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f((m - m_new) * LOG2E);
+    float psum = 0.f;
+#pragma unroll
+    for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = (sc[jt][i] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((sc[jt][i] - m_new) * LOG2E);
+        sc[jt][i] = p;
+        psum += p;
+      }
+    l = l * alpha + psum;
+    m = m_new;
+    // ---- U^T = U^T alpha + C^T P^T
+    const bf16x8 pb = __builtin_bit_cast(bf16x8, make_uint4(pack_bf16(sc[0][0], sc[0][1]), pack_bf16(sc[0][2], sc[0][3]),
+                                                            pack_bf16(sc[1][0], sc[1][1]), pack_bf16(sc[1][2], sc[1][3])));
+#pragma unroll
+    for (int t = 0; t < VT; ++t)
+      if (EXACT || t < vt) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[t][i] *= alpha;
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(vts + (16 * t + r) * LM_VROW + 8 * kb),
+                                                       pb, o[t], 0, 0, 0);
+      }
+  }
+  if (!working) return;
+  l += __shfl_xor(l, 16, QIL_WAVE);
+  l += __shfl_xor(l, 32, QIL_WAVE);
+  if (!valid) return;
+  if (parts == 1) {
+    const float inv = 1.f / l;
+    float* dst = out + gcol * rank + 4 * kb;
+#pragma unroll
+    for (int t = 0; t < VT; ++t)
+      if (EXACT || t < vt)
+        *reinterpret_cast<float4*>(dst + 16 * t) = make_float4(o[t][0] * inv, o[t][1] * inv, o[t][2] * inv, o[t][3] * inv);
+    return;
+  }
+  const size_t cell = gcol * parts + part;
+  if (kb == 0) {
+    part_m[cell] = m;
+    part_l[cell] = l;
+  }
+  float* dst = part_acc + cell * rank + 4 * kb;
+#pragma unroll
+  for (int t = 0; t < VT; ++t)
+    if (EXACT || t < vt) *reinterpret_cast<float4*>(dst + 16 * t) = make_float4(o[t][0], o[t][1], o[t][2], o[t][3]);
+}
+
+// out[column] = sum_p w_p acc_p / (sum_p w_p l_p + exp(sink - M)), w_p = exp(m_p - M), M the largest of the parts' maxima
+// and the sink, over the parts that the row's position reaches.  One block per (row, head).
+__global__ void latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_m,
+                                    const float* __restrict__ part_l, const int* __restrict__ positions,
+                                    const float* __restrict__ sink, float* __restrict__ out, int heads, int rank, int P,
+                                    int parts) {
+  const int n = blockIdx.x, h = blockIdx.y;
+  const size_t column = (size_t)n * heads + h;
+  const int reached = min(parts, positions[n] / P + 1);
+  const float floor_ = sink ? sink[h] : -INFINITY;
+  float top = floor_;
+  for (int p = 0; p < reached; ++p) top = fmaxf(top, part_m[column * parts + p]);
+  float below = sink ? expf(floor_ - top) : 0.f;
+  for (int p = 0; p < reached; ++p) {
+    const float mp = part_m[column * parts + p];
+    if (mp > -INFINITY) below += expf(mp - top) * part_l[column * parts + p];
+  }
+  for (int c = threadIdx.x; c < rank; c += blockDim.x) {
+    float acc = 0.f;
+    for (int p = 0; p < reached; ++p) {
+      const float mp = part_m[column * parts + p];
+      if (mp > -INFINITY) acc += expf(mp - top) * part_acc[(column * parts + p) * rank + c];
+    }
+    out[column * rank + c] = acc / below;
+  }
+}
+
+static int lm_lds_bytes(int rank, int rot) {
+  const int dp = (rank + rot + 31) / 32 * 32;
+  return (LM_KEYS * (dp + 8) + rank * LM_VROW) * (int)sizeof(bf16_t);
+}
+
+template <int QF, int VT, bool EXACT>
+static int lm_launch(dim3 grid, size_t lds, hipStream_t s, const float* q, const bf16_t* latent, const bf16_t* rope,
+                     const int* tables, int table_stride, const int* cu_seqlens, const int* seq_starts, int n_seqs,
+                     int single, const float* sink, float* out, float* part_acc, float* part_m, float* part_l, int heads,
+                     int rank, int rot, int page_size, float scale, int rt, int hb, int P, int parts) {
+  auto kernel = latent_mfma_kernel<QF, VT, EXACT>;
+  static bool raised = false;                                // per instantiation
+  if (lds > 64 * 1024 && !raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return (int)e;
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(LM_THREADS), lds, s, q, latent, rope, tables, table_stride, cu_seqlens, seq_starts,
+                     n_seqs, single, sink, out, part_acc, part_m, part_l, heads, rank, rot, page_size, scale, rt, hb, P,
+                     parts);
+  return 0;
+}
+
+extern "C" {
+
+int qil_latent_mfma_takes(int heads, int rank, int rot) {
+  return heads >= 1 && rank >= 16 && rank % 16 == 0 && rot >= 0 && rot % 8 == 0 && rank + rot <= 640 && rank <= 512 &&
+         lm_lds_bytes(rank, rot) <= 160 * 1024;
+}
+
+// (rows a block, heads a block, keys a part, parts) for a step: blocks of up to 64 columns; the keys in parts of at
+// least 128 while the blocks are fewer than two a compute unit.
+void qil_latent_mfma_plan(int n_rows, int n_seqs, int single, int heads, int max_context, int* rt, int* hb, int* P,
+                          int* parts) {
+  *hb = heads < 64 ? heads : 64;
+  *rt = single ? 1 : (64 / *hb > 0 ? 64 / *hb : 1);
+  const int tiles = single ? n_seqs : (n_rows + *rt - 1) / *rt + n_seqs;
+  const long blocks = (long)tiles * ((heads + *hb - 1) / *hb);
+  int want = (int)((2 * QIL_CUS + blocks - 1) / blocks);
+  if (want < 1) want = 1;
+  int part = ((max_context + want - 1) / want + 31) / 32 * 32;
+  if (part < 128) part = 128;
+  *P = part;
+  *parts = (max_context + part - 1) / part;
+  if (*parts < 1) *parts = 1;
+}
+
+size_t qil_latent_mfma_workspace(int n_rows, int heads, int rank, int parts) {
+  return parts > 1 ? (size_t)n_rows * heads * parts * (rank + 2) * sizeof(float) : 0;
+}
+
+// q float32 [n_rows, heads, rank + rot]; out float32 [n_rows, heads, rank]; workspace as qil_latent_mfma_workspace says.
+// single: every sequence has one row (n_seqs == n_rows).  rt, hb, P, parts: as qil_latent_mfma_plan gave them.
+int qil_latent_mfma(const float* q, const void* latent, const void* rope, const int* tables, int table_stride,
+                    const int* cu_seqlens, const int* seq_starts, const int* positions, const float* sink, float* out,
+                    float* workspace, int n_rows, int n_seqs, int single, int heads, int rank, int rot, int page_size,
+                    float scale, int rt, int hb, int P, int parts, hipStream_t s) {
+  if (n_rows == 0) return 0;
+  if (!qil_latent_mfma_takes(heads, rank, rot) || page_size < 1 || rt < 1 || hb < 1 || rt * hb > 64 || P < 32 || P % 32 ||
+      parts < 1 || (single && n_seqs != n_rows) || (parts > 1 && !workspace))
+    return -1;
+  const int tiles = single ? n_seqs : (n_rows + rt - 1) / rt + n_seqs;
+  dim3 grid(tiles, (heads + hb - 1) / hb, parts);
+  const size_t lds = (size_t)lm_lds_bytes(rank, rot);
+  float* part_acc = workspace;
+  float* part_m = parts > 1 ? workspace + (size_t)n_rows * heads * parts * rank : nullptr;
+  float* part_l = parts > 1 ? part_m + (size_t)n_rows * heads * parts : nullptr;
+  const int qf = (rank + rot + 31) / 32, vt = rank / 16;
+  int status;
+#define QIL_LM(QF, VT, EXACT)                                                                                         \
+  status = lm_launch<QF, VT, EXACT>(grid, lds, s, q, (const bf16_t*)latent, (const bf16_t*)rope, tables, table_stride, \
+                                    cu_seqlens, seq_starts, n_seqs, single, parts == 1 ? sink : nullptr, out, part_acc, \
+                                    part_m, part_l, heads, rank, rot, page_size, scale, rt, hb, P, parts)
+  if (qf == 18 && vt == 32) QIL_LM(18, 32, true);
+  else if (qf == 5 && vt == 8) QIL_LM(5, 8, true);
+  else if (qf <= 8 && vt <= 8) QIL_LM(8, 8, false);
+  else if (qf <= 12 && vt <= 16) QIL_LM(12, 16, false);
+  else QIL_LM(20, 32, false);
+#undef QIL_LM
+  if (status) return status;
+  if (parts > 1)
+    hipLaunchKernelGGL(latent_merge_kernel, dim3(n_rows, heads), dim3(rank >= 256 ? 256 : 64), 0, s, part_acc, part_m,
+                       part_l, positions, sink, out, heads, rank, P, parts);
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+}  // extern "C"

@@ -863,12 +863,22 @@ def latent_query(q, k_up, *, heads, dim, rot, rank, frequencies, positions):
     return out
 
 
-def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, positions, sink, scale, heads, rank, rot):
+# False: bfloat16 caches go to the general kernel too (tests and tuning runs).
+LATENT_MATRIX_CORES = True
+LATENT_KEY_PARTS = None     # tests: (keys a part, parts) forces the matrix-core kernel's split of the keys
+
+
+def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, positions, sink, scale, heads, rank, rot,
+                     cu_seqlens=None, seq_starts=None, n_seqs=None, max_query=None, max_context=None):
     """Every row's attention over its request's cached latents: ``q`` float32 [N, heads * (rank + rot)] as
     ``latent_query`` makes it; caches [pages, page_size, rank] and [pages, page_size, rot]; row n sees keys
     j <= positions[n] of sequence row_seq[n] (a row of ``block_tables``).  ``sink`` float32 [heads] or None: a logit
     per head that counts once in the softmax's denominator and has no value.  -> float32 [N, heads * rank], the
-    weighted sums of the latents."""
+    weighted sums of the latents.
+
+    With the step's description (``cu_seqlens``, ``seq_starts``, ``n_seqs``, ``max_query``, ``max_context``; rows packed
+    sequence after sequence) bfloat16 caches of sizes it takes go to the matrix-core kernel, which serves several rows
+    and all heads from one staged tile of keys and cuts the keys into parts when the step has few rows."""
     n = q.shape[0]
     _require(q, 'q', torch.float32, (n, heads * (rank + rot)))
     _require(latent, 'latent')
@@ -885,6 +895,25 @@ def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, posit
     if not lib.qil_latent_attention_takes(heads, rank, rot):
         raise UnsupportedShape(f'latent attention: {heads} heads, rank {rank}, {rot} rotated elements')
     out = torch.empty((n, heads * rank), dtype=torch.float32, device=q.device)
+    if LATENT_MATRIX_CORES and latent.dtype == torch.bfloat16 and cu_seqlens is not None and \
+            lib.qil_latent_mfma_takes(heads, rank, rot):
+        _require(cu_seqlens, 'cu_seqlens', torch.int32, (n_seqs + 1,))
+        _require(seq_starts, 'seq_starts', torch.int32, (n_seqs,))
+        if block_tables.shape[0] != n_seqs or block_tables.shape[1] * page_size < max_context:
+            raise ValueError('one block table row per sequence, wide enough for the longest context')
+        single = int(max_query == 1)
+        plan = [ctypes.c_int(0) for _ in range(4)]
+        lib.qil_latent_mfma_plan(n, n_seqs, single, heads, max_context, *[ctypes.byref(v) for v in plan])
+        rt, hb, part, parts = (v.value for v in plan)
+        if LATENT_KEY_PARTS is not None:
+            part, parts = LATENT_KEY_PARTS[0], max(LATENT_KEY_PARTS[1], -(-max_context // LATENT_KEY_PARTS[0]))
+        nbytes = lib.qil_latent_mfma_workspace(n, heads, rank, parts)
+        workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=q.device) if nbytes else None
+        _check(lib.qil_latent_mfma(_ptr(q), _ptr(latent), _ptr(rope), _ptr(block_tables), block_tables.shape[1],
+                                   _ptr(cu_seqlens), _ptr(seq_starts), _ptr(positions), _ptr(sink), _ptr(out),
+                                   _ptr(workspace), n, n_seqs, single, heads, rank, rot, page_size, float(scale), rt, hb,
+                                   part, parts, _stream()), 'latent_mfma')
+        return out
     _check(lib.qil_latent_attention(_ptr(q), _ptr(latent), _ptr(rope), _ptr(block_tables), block_tables.shape[1],
                                     _ptr(row_seq), _ptr(positions), _ptr(sink), _ptr(out), n, heads, rank, rot, page_size,
                                     float(scale), _code(latent.dtype), _stream()), 'latent_attention')

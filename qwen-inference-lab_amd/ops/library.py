@@ -295,6 +295,15 @@ def _declare(lib):
     lib.qil_latent_attention_takes.argtypes = [i, i, i]
     lib.qil_latent_attention_takes.restype = i
     lib.qil_latent_attention.argtypes = [p, p, p, p, i, p, p, p, p, i, i, i, i, i, f, i, p]
+    lib.qil_latent_mfma_takes.argtypes = [i, i, i]
+    lib.qil_latent_mfma_takes.restype = i
+    ip = ctypes.POINTER(ctypes.c_int)
+    lib.qil_latent_mfma_plan.argtypes = [i, i, i, i, i, ip, ip, ip, ip]
+    lib.qil_latent_mfma_plan.restype = None
+    lib.qil_latent_mfma_workspace.argtypes = [i, i, i, i]
+    lib.qil_latent_mfma_workspace.restype = z
+    lib.qil_latent_mfma.argtypes = [p, p, p, p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, i, i, p]
+    lib.qil_latent_mfma.restype = i
     lib.qil_state_scan_slot.argtypes = [i, i, i, i]
     lib.qil_state_scan_slot.restype = z
     lib.qil_state_scan_takes.argtypes = [i, i, i]

@@ -76,6 +76,8 @@ class LatentAttention(Mixer):
         mixed = ops.latent_attention(q, latent=cache.tensors['latent'], rope=cache.tensors['rope'],
                                      page_size=cache.page_size, block_tables=cache.block_tables, row_seq=ctx.row_seq,
                                      positions=ctx.positions, sink=p.get('sink'), scale=self.scale, heads=self.heads,
-                                     rank=self.kv_rank, rot=self.rot_dim)
+                                     rank=self.kv_rank, rot=self.rot_dim, cu_seqlens=ctx.cu_seqlens,
+                                     seq_starts=ctx.seq_starts, n_seqs=ctx.n_seqs, max_query=ctx.max_query,
+                                     max_context=ctx.max_context)
         values = ops.head_product(mixed, p['v_up.weight'], heads=self.heads, out_dtype=self.dtype)
         return ops.linear(values, p['o_proj.weight'], None, partials=True)

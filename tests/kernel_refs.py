@@ -215,7 +215,8 @@ def latent_query(q, k_up, *, heads, dim, rot, rank, frequencies, positions):
     return torch.cat([absorbed, _turn(q[:, :, dim:], positions, frequencies)], dim=-1).reshape(n, heads * (rank + rot))
 
 
-def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, positions, sink, scale, heads, rank, rot):
+def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, positions, sink, scale, heads, rank, rot,
+                     **step):
     n = q.shape[0]
     q = q.view(n, heads, rank + rot)
     out = torch.zeros((n, heads, rank), dtype=torch.float32)

@@ -273,3 +273,47 @@ def test_head_norm_and_gate(dtype):
                                  weight=None if w is None else w.cuda(), eps=1e-5, gate=gate, out_dtype=dtype)
         close(got, refs.head_norm_gate(o, source, gate_offset=10, heads=heads, vdim=vdim, weight=w, eps=1e-5, gate=gate,
                                        out_dtype=dtype), dtype, 3.0)
+
+
+@pytest.mark.parametrize('sizes', [dict(heads=5, rank=32, rot=8, page=4), dict(heads=6, rank=128, rot=32, page=16),
+                                   dict(heads=16, rank=512, rot=64, page=16), dict(heads=70, rank=48, rot=16, page=8)])
+@pytest.mark.parametrize('step', ['portions', 'single rows', 'both'])
+@pytest.mark.parametrize('key_parts', [None, (64, 1), (32, 3)])
+def test_latent_attention_on_the_matrix_cores(sizes, step, key_parts, monkeypatch):
+    """bfloat16 caches with the step's description: sequences of several rows (tiles of rows that share staged keys,
+    starting at any position), rows alone in their sequences, the keys in one piece and in parts."""
+    heads, rank, rot, page = sizes['heads'], sizes['rank'], sizes['rot'], sizes['page']
+    g = torch.Generator().manual_seed(rank + heads)
+    lengths = {'portions': [(130, 41), (0, 67), (63, 2)], 'single rows': [(200, 1), (0, 1), (64, 1), (31, 1)],
+               'both': [(95, 33), (17, 3), (150, 1), (0, 1)]}[step]                # (tokens cached before, rows of the step)
+    most = max(a + b for a, b in lengths)
+    pages_each = -(-most // page)
+    order = torch.randperm(pages_each * len(lengths) + 2, generator=g)
+    latent = torch.full((len(order), page, rank), float('nan')).to(torch.bfloat16)
+    rope = torch.full((len(order), page, rot), float('nan')).to(torch.bfloat16)
+    tables = order[:pages_each * len(lengths)].view(len(lengths), pages_each).to(torch.int32)
+    positions, row_seq, cu = [], [], [0]
+    for s, (cached, rows) in enumerate(lengths):
+        keys = torch.arange(cached + rows)
+        slots = tables[s].long()[keys // page] * page + keys % page
+        latent.view(-1, rank)[slots] = torch.randn(len(keys), rank, generator=g).to(torch.bfloat16)
+        rope.view(-1, rot)[slots] = torch.randn(len(keys), rot, generator=g).to(torch.bfloat16)
+        positions += list(range(cached, cached + rows))
+        row_seq += [s] * rows
+        cu.append(cu[-1] + rows)
+    n = len(positions)
+    positions, row_seq, cu = (torch.tensor(v, dtype=torch.int32) for v in (positions, row_seq, cu))
+    starts = torch.tensor([a for a, _ in lengths], dtype=torch.int32)
+    q = torch.randn(n, heads * (rank + rot), generator=g) * 0.4
+    sink = torch.randn(heads, generator=g)
+    monkeypatch.setattr(ops, 'LATENT_KEY_PARTS', key_parts)
+    for s in (sink, None):
+        common = dict(page_size=page, scale=(rank + rot) ** -0.5 * 3, heads=heads, rank=rank, rot=rot)
+        want = refs.latent_attention(q, latent=latent, rope=rope, block_tables=tables, row_seq=row_seq, positions=positions,
+                                     sink=s, **common)
+        got = ops.latent_attention(q.cuda(), latent=latent.cuda(), rope=rope.cuda(), block_tables=tables.cuda(),
+                                   row_seq=row_seq.cuda(), positions=positions.cuda(), sink=None if s is None else s.cuda(),
+                                   cu_seqlens=cu.cuda(), seq_starts=starts.cuda(), n_seqs=len(lengths),
+                                   max_query=max(b for _, b in lengths), max_context=most, **common)
+        assert torch.isfinite(got).all()
+        torch.testing.assert_close(got.cpu(), want, atol=2e-2, rtol=2e-2)          # queries and probabilities are rounded to bfloat16
