@@ -927,9 +927,10 @@ SCAN_MODES = {'decay': 0, 'mlstm': 1}
 
 def state_scan_slot(*, heads, dim, vdim, mode):
     """float32 elements of one request's state for ``state_scan``: the heads' [dim, vdim] matrices, and for 'mlstm' a
-    normaliser [dim] and a maximum per head and tile of 64 state columns (the kernel's blocks keep one each)."""
-    tiles = -(-vdim // 64)
-    return heads * dim * vdim + (heads * tiles * (dim + 1) if SCAN_MODES[mode] == SCAN_MODES['mlstm'] else 0)
+    normaliser [dim] per head and the running maximum once per head and block of the kernel (one per 16 state columns
+    and one for the normaliser's)."""
+    tiles = -(-vdim // 16)
+    return heads * dim * vdim + (heads * (dim + tiles + 1) if SCAN_MODES[mode] == SCAN_MODES['mlstm'] else 0)
 
 
 def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, state, cu_seqlens, seq_starts, seq_slots,
@@ -941,7 +942,9 @@ def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, st
     and values from ``v_offset`` (heads * vdim).  Mode 'decay': a_t = decay[h], b_t = 1.  Mode 'mlstm': exponential
     gates from ``gates`` float32 [N, 2 heads] (+ ``gate_bias`` [2 heads]; input gates first) soft-capped at ``cap``,
     with a running maximum and a normaliser.  Queries and keys are rotated by position on their leading ``rot``
-    elements (``frequencies`` [rot / 2]) and then scaled.  -> float32 [N, heads * vdim]."""
+    elements (``frequencies`` [rot / 2]) and then scaled.
+    -> (float32 [N, heads * vdim], denominators): 'decay' gives o_t and None; 'mlstm' gives S_t^T q_t undivided and
+    float32 [N, heads] with max(|n_t . q_t|, exp(-m_t)) + 1e-6, which ``head_norm_gate`` divides by."""
     n = proj.shape[0]
     _require(proj, 'proj')
     code = _code(proj.dtype)
@@ -968,17 +971,21 @@ def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, st
     if rot:
         _require(frequencies, 'frequencies', torch.float32, (rot // 2,))
     out = torch.empty((n, heads * vdim), dtype=torch.float32, device=proj.device)
+    below = torch.empty((n, heads), dtype=torch.float32, device=proj.device) if mode == 'mlstm' else None
     _check(lib.qil_state_scan(_ptr(proj), code, width, q_offset, k_offset, v_offset, _ptr(gates), _ptr(gate_bias),
                               float(cap), _ptr(decay), _ptr(frequencies) if rot else None, rot, float(q_scale),
                               float(k_scale), _ptr(state), _ptr(cu_seqlens), _ptr(seq_starts), _ptr(seq_slots), _ptr(out),
-                              n_seqs, heads, dim, vdim, SCAN_MODES[mode], _stream()), 'state_scan')
-    return out
+                              _ptr(below), n_seqs, heads, dim, vdim, SCAN_MODES[mode], _stream()), 'state_scan')
+    return out, below
 
 
-def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gate, out_dtype):
-    """Per head: o / sqrt(mean(o^2) + eps) (* weight) * act(g), ``o`` float32 [N, heads * vdim], g the heads * vdim
-    columns of ``gate_source`` from ``gate_offset``; ``gate``: 'sigmoid' or 'silu'.  -> [N, heads * vdim] out_dtype."""
+def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gate, out_dtype, denominators=None):
+    """Per head: o / sqrt(mean(o^2) + eps) (* weight) * act(g), ``o`` float32 [N, heads * vdim] (first divided, head by
+    head, by ``denominators`` float32 [N, heads] if given), g the heads * vdim columns of ``gate_source`` from
+    ``gate_offset``; ``gate``: 'sigmoid' or 'silu'.  -> [N, heads * vdim] out_dtype."""
     n = o.shape[0]
+    if denominators is not None:
+        _require(denominators, 'denominators', torch.float32, (n, heads))
     _require(o, 'o', torch.float32, (n, heads * vdim))
     _require(gate_source, 'gate_source', out_dtype)
     if gate_source.shape[0] != n or gate_offset + heads * vdim > gate_source.shape[1]:
@@ -986,7 +993,7 @@ def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gat
     if weight is not None:
         _require(weight, 'weight', torch.float32, (heads * vdim,))
     out = torch.empty((n, heads * vdim), dtype=out_dtype, device=o.device)
-    _check(library.load().qil_head_norm_gate(_ptr(o), _ptr(gate_source), gate_source.shape[1], gate_offset, _ptr(weight),
+    _check(library.load().qil_head_norm_gate(_ptr(o), _ptr(denominators), _ptr(gate_source), gate_source.shape[1], gate_offset, _ptr(weight),
                                              _ptr(out), n, heads, vdim, float(eps), {'sigmoid': 0, 'silu': 1}[gate],
                                              _code(out_dtype), _stream()), 'head_norm_gate')
     return out

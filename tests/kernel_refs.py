@@ -235,19 +235,21 @@ def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, posit
 
 
 def state_scan_slot(*, heads, dim, vdim, mode):
-    tiles = -(-vdim // 64)
-    return heads * dim * vdim + (heads * tiles * (dim + 1) if mode == 'mlstm' else 0)
+    tiles = -(-vdim // 16)
+    return heads * dim * vdim + (heads * (dim + tiles + 1) if mode == 'mlstm' else 0)
 
 
 def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, state, cu_seqlens, seq_starts, seq_slots,
                n_seqs, gates=None, gate_bias=None, cap=0.0, decay=None, frequencies=None, rot=0, q_scale=1.0, k_scale=1.0):
-    """The state slot's layout is the kernel's: matrices, then per head and tile of 64 columns a normaliser and a maximum."""
-    n, tiles = proj.shape[0], -(-vdim // 64)
+    """-> (o, denominators): for 'mlstm' o is undivided and the denominators are returned beside it.  The state slot's
+    layout is the kernel's: matrices, then a normaliser per head, then the maximum tiles + 1 times per head."""
+    n, tiles = proj.shape[0], -(-vdim // 16)
     x = proj.to(torch.float32)
     q = x[:, q_offset:q_offset + heads * dim].reshape(n, heads, dim).clone()
     k = x[:, k_offset:k_offset + heads * dim].reshape(n, heads, dim).clone()
     v = x[:, v_offset:v_offset + heads * vdim].reshape(n, heads, vdim)
     out = torch.zeros((n, heads, vdim), dtype=torch.float32)
+    below = torch.zeros((n, heads), dtype=torch.float32) if mode == 'mlstm' else None
     mats = heads * dim * vdim
     for s in range(n_seqs):
         lo, hi, start, slot = int(cu_seqlens[s]), int(cu_seqlens[s + 1]), int(seq_starts[s]), int(seq_slots[s])
@@ -260,9 +262,9 @@ def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, st
         fresh = start == 0
         memory = torch.zeros(heads, dim, vdim) if fresh else state[slot, :mats].view(heads, dim, vdim).clone()
         if mode == 'mlstm':
-            norms = state[slot, mats:mats + heads * tiles * dim].view(heads, tiles, dim)
-            tops = state[slot, mats + heads * tiles * dim:].view(heads, tiles)
-            norm = torch.zeros(heads, dim) if fresh else norms[:, 0].clone()
+            norms = state[slot, mats:mats + heads * dim].view(heads, dim)
+            tops = state[slot, mats + heads * dim:].view(heads, tiles + 1)
+            norm = torch.zeros(heads, dim) if fresh else norms.clone()
             top = torch.zeros(heads) if fresh else tops[:, 0].clone()
         for t in range(hi - lo):
             if mode == 'mlstm':
@@ -277,18 +279,20 @@ def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, st
             read = torch.einsum('hdv,hd->hv', memory, qs[t])
             if mode == 'mlstm':
                 norm = a[:, None] * norm + b[:, None] * ks[t]
-                read = read / (torch.maximum((norm * qs[t]).sum(-1).abs(), torch.exp(-top)) + 1e-6)[:, None]
+                below[lo + t] = torch.maximum((norm * qs[t]).sum(-1).abs(), torch.exp(-top)) + 1e-6
             out[lo + t] = read
         state[slot, :mats] = memory.reshape(-1)
         if mode == 'mlstm':
-            norms[:] = norm[:, None, :]
+            norms[:] = norm
             tops[:] = top[:, None]
-    return out.reshape(n, heads * vdim)
+    return out.reshape(n, heads * vdim), below
 
 
-def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gate, out_dtype):
+def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gate, out_dtype, denominators=None):
     n = o.shape[0]
     unit = o.view(n, heads, vdim)
+    if denominators is not None:
+        unit = unit / denominators[:, :, None]
     unit = (unit / torch.sqrt(unit.square().mean(dim=-1, keepdim=True) + eps)).reshape(n, heads * vdim)
     if weight is not None:
         unit = unit * weight
