@@ -923,6 +923,7 @@ def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, posit
 # ---------------------------------------------------------------------------------------------------------------
 # Recurrences with a matrix state
 SCAN_MODES = {'decay': 0, 'mlstm': 1}
+SCAN_BLOCKS_FROM = 32           # rows of one sequence from which a step's recurrence runs in blocks side by side
 
 
 def state_scan_slot(*, heads, dim, vdim, mode):
@@ -934,7 +935,8 @@ def state_scan_slot(*, heads, dim, vdim, mode):
 
 
 def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, state, cu_seqlens, seq_starts, seq_slots,
-               n_seqs, gates=None, gate_bias=None, cap=0.0, decay=None, frequencies=None, rot=0, q_scale=1.0, k_scale=1.0):
+               n_seqs, gates=None, gate_bias=None, cap=0.0, decay=None, frequencies=None, rot=0, q_scale=1.0, k_scale=1.0,
+               max_query=None):
     """S_t = a_t S_(t-1) + b_t k_t v_t^T, o_t = S_t^T q_t per head over every sequence's rows of the step, from the
     sequence's state slot (empty where the sequence starts at position 0) and back into it.
 
@@ -942,7 +944,9 @@ def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, st
     and values from ``v_offset`` (heads * vdim).  Mode 'decay': a_t = decay[h], b_t = 1.  Mode 'mlstm': exponential
     gates from ``gates`` float32 [N, 2 heads] (+ ``gate_bias`` [2 heads]; input gates first) soft-capped at ``cap``,
     with a running maximum and a normaliser.  Queries and keys are rotated by position on their leading ``rot``
-    elements (``frequencies`` [rot / 2]) and then scaled.
+    elements (``frequencies`` [rot / 2]) and then scaled.  ``max_query``: the most rows of one sequence, if the caller
+    knows it; from ``SCAN_BLOCKS_FROM`` rows on the step is worked in blocks of 64 tokens side by side (the sums of the
+    blocks, their carry from block to block, the outputs), below that token by token.
     -> (float32 [N, heads * vdim], denominators): 'decay' gives o_t and None; 'mlstm' gives S_t^T q_t undivided and
     float32 [N, heads] with max(|n_t . q_t|, exp(-m_t)) + 1e-6, which ``head_norm_gate`` divides by."""
     n = proj.shape[0]
@@ -972,6 +976,16 @@ def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, st
         _require(frequencies, 'frequencies', torch.float32, (rot // 2,))
     out = torch.empty((n, heads * vdim), dtype=torch.float32, device=proj.device)
     below = torch.empty((n, heads), dtype=torch.float32, device=proj.device) if mode == 'mlstm' else None
+    if max_query is not None and max_query >= SCAN_BLOCKS_FROM:
+        floats = lib.qil_state_scan_chunked_workspace(n, n_seqs, heads, dim, vdim, SCAN_MODES[mode])
+        workspace = torch.empty(floats, dtype=torch.float32, device=proj.device)
+        _check(lib.qil_state_scan_chunked(_ptr(proj), code, width, q_offset, k_offset, v_offset, _ptr(gates),
+                                          _ptr(gate_bias), float(cap), _ptr(decay), _ptr(frequencies) if rot else None,
+                                          rot, float(q_scale), float(k_scale), _ptr(state), slot, _ptr(cu_seqlens),
+                                          _ptr(seq_starts), _ptr(seq_slots), _ptr(out), _ptr(below), _ptr(workspace), n,
+                                          n_seqs, int(max_query), heads, dim, vdim, SCAN_MODES[mode], _stream()),
+               'state_scan_chunked')
+        return out, below
     _check(lib.qil_state_scan(_ptr(proj), code, width, q_offset, k_offset, v_offset, _ptr(gates), _ptr(gate_bias),
                               float(cap), _ptr(decay), _ptr(frequencies) if rot else None, rot, float(q_scale),
                               float(k_scale), _ptr(state), _ptr(cu_seqlens), _ptr(seq_starts), _ptr(seq_slots), _ptr(out),

@@ -310,6 +310,10 @@ def _declare(lib):
     lib.qil_state_scan_takes.restype = i
     lib.qil_state_scan.argtypes = [p, i, i, i, i, i, p, p, f, p, p, i, f, f, p, p, p, p, p, p, i, i, i, i, i, p]
     lib.qil_head_norm_gate.argtypes = [p, p, p, i, i, p, p, i, i, i, f, i, i, p]
+    lib.qil_state_scan_chunked_workspace.argtypes = [i, i, i, i, i, i]
+    lib.qil_state_scan_chunked_workspace.restype = z
+    lib.qil_state_scan_chunked.argtypes = [p, i, i, i, i, i, p, p, f, p, p, i, f, f, p, z, p, p, p, p, p, p, i, i, i, i, i, i, i, p]
+    lib.qil_state_scan_chunked.restype = i
     for name in ('qil_add_norm', 'qil_gated_act', 'qil_latent_prepare', 'qil_head_product', 'qil_rotate_tail',
                  'qil_latent_attention', 'qil_state_scan', 'qil_head_norm_gate'):
         getattr(lib, name).restype = i

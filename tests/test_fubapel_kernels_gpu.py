@@ -189,9 +189,12 @@ def scan_inputs(dtype, g, *, n, heads, dim, vdim):
 @pytest.mark.parametrize('mode', ['decay', 'mlstm'])
 @pytest.mark.parametrize('sizes', [dict(heads=2, dim=24, vdim=16, rot=8), dict(heads=3, dim=72, vdim=130, rot=72),
                                    dict(heads=1, dim=200, vdim=64, rot=0), dict(heads=2, dim=5, vdim=3, rot=2)])
-def test_state_scan_against_the_reference(dtype, mode, sizes):
+@pytest.mark.parametrize('steps', [pytest.param((([4, 1, 9], [7, 0, 0]), ([1, 6, 2], [11, 1, 9])), id='token-by-token'),
+                                   pytest.param((([130, 1, 64], [7, 0, 0]), ([65, 200, 2], [137, 1, 64])), id='blocks')])
+def test_state_scan_against_the_reference(dtype, mode, sizes, steps):
     """Three sequences in one step (one continues from a state, two begin; slots out of order and one used before),
-    then a second step that continues all of them with other lengths."""
+    then a second step that continues all of them with other lengths.  With long sequences the step runs in blocks of
+    tokens side by side: whole blocks, a block of one token, sequences that end inside a block."""
     heads, dim, vdim, rot = sizes['heads'], sizes['dim'], sizes['vdim'], sizes['rot']
     g = torch.Generator().manual_seed(dim)
     slot = ops.state_scan_slot(heads=heads, dim=dim, vdim=vdim, mode=mode)
@@ -209,8 +212,9 @@ def test_state_scan_against_the_reference(dtype, mode, sizes):
         extra_c.update(gate_bias=bias, cap=6.0)
     else:
         extra_c.update(decay=torch.tensor([0.9, 0.99, 0.999][:heads]))
-    for counts, starts in (([4, 1, 9], [7, 0, 0]), ([1, 6, 2], [11, 1, 9])):
+    for counts, starts in steps:
         n = sum(counts)
+        assert (max(counts) >= ops.SCAN_BLOCKS_FROM) == (max(counts) > 9)
         proj, where = scan_inputs(dtype, g, n=n, heads=heads, dim=dim, vdim=vdim)
         cu = torch.tensor([0] + torch.tensor(counts).cumsum(0).tolist(), dtype=torch.int32)
         st, sl = torch.tensor(starts, dtype=torch.int32), torch.tensor([3, 0, 4], dtype=torch.int32)
@@ -221,7 +225,7 @@ def test_state_scan_against_the_reference(dtype, mode, sizes):
         want = refs.state_scan(proj, mode=mode, state=state_c, cu_seqlens=cu, seq_starts=st, seq_slots=sl, n_seqs=3,
                                **where, **step_c)
         got = ops.state_scan(proj.cuda(), mode=mode, state=state_g, cu_seqlens=cu.cuda(), seq_starts=st.cuda(),
-                             seq_slots=sl.cuda(), n_seqs=3, **where, **step_g)
+                             seq_slots=sl.cuda(), n_seqs=3, max_query=max(counts), **where, **step_g)
         close(got[0], want[0], torch.float32, max(1.0, want[0].abs().max().item()))
         if mode == 'mlstm':
             close(got[1], want[1], torch.float32, max(1.0, want[1].abs().max().item()))
