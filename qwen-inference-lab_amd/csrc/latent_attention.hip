@@ -79,6 +79,63 @@ __global__ void head_product_kernel(const TX* __restrict__ x, int x_row, int x_h
     if (row0 + r < n_rows) st(out + (size_t)(row0 + r) * out_row + (size_t)h * out_head + o, acc[r]);
 }
 
+// The same product for few rows (decoding): the weights of a head are then read by too few blocks for the chip, so a
+// block takes 8 rows, 64 outputs and splits k 32 ways: a thread reads 8 consecutive outputs of every 32nd k (16 bytes
+// of bfloat16), and the 32 partial sums meet by shuffles in a wave and through LDS between the four waves.
+// Takes o_dim % 8 == 0 and w aligned to 8 elements.
+template <typename TX, typename TW, typename TO>
+__global__ void __launch_bounds__(256)
+head_product_few_kernel(const TX* __restrict__ x, int x_row, int x_head, const TW* __restrict__ w, TO* __restrict__ out,
+                        int out_row, int out_head, int n_rows, int k_dim, int o_dim) {
+  extern __shared__ float xs[];                       // [8][k_dim], then [4 waves][8 rows][64 outputs]
+  float* sums = xs + 8 * k_dim;
+  const int row0 = blockIdx.x * 8, h = blockIdx.y, tid = threadIdx.x, to = tid & 7, kg = tid >> 3;
+  const int o0 = blockIdx.z * 64 + to * 8;
+  for (int idx = tid; idx < 8 * k_dim; idx += 256) {
+    const int r = idx / k_dim, k = idx - r * k_dim;
+    xs[idx] = row0 + r < n_rows ? ld(x + (size_t)(row0 + r) * x_row + (size_t)h * x_head + k) : 0.f;
+  }
+  __syncthreads();
+  float acc[8][8] = {};
+  if (o0 < o_dim) {
+    const TW* wh = w + (size_t)h * k_dim * o_dim + o0;
+    for (int k = kg; k < k_dim; k += 32) {
+      float wv[8];
+      ld8(wh + (size_t)k * o_dim, wv);
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const float xv = xs[r * k_dim + k];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[r][j] += xv * wv[j];
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 8; ++r)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float v = acc[r][j];
+      v += __shfl_xor(v, 8, QIL_WAVE);
+      v += __shfl_xor(v, 16, QIL_WAVE);
+      v += __shfl_xor(v, 32, QIL_WAVE);
+      acc[r][j] = v;
+    }
+  const int wave = tid >> 6;
+  if ((tid & 63) < 8) {
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sums[(wave * 8 + r) * 64 + to * 8 + j] = acc[r][j];
+  }
+  __syncthreads();
+  for (int idx = tid; idx < 8 * 64; idx += 256) {
+    const int r = idx / 64, j = idx % 64, o = blockIdx.z * 64 + j;
+    if (row0 + r < n_rows && o < o_dim)
+      st(out + (size_t)(row0 + r) * out_row + (size_t)h * out_head + o,
+         sums[r * 64 + j] + sums[(8 + r) * 64 + j] + sums[(16 + r) * 64 + j] + sums[(24 + r) * 64 + j]);
+  }
+}
+
 // The rotated tail of every head's query: out[n, h, i] = rotate(q[n, h, offset + i], position), i < rot.
 template <typename TX>
 __global__ void rotate_tail_kernel(const TX* __restrict__ q, int q_row, int q_head, int offset, const float* __restrict__ freq,
@@ -240,9 +297,18 @@ int qil_head_product(const void* x, int x_dtype, int x_row, int x_head, const vo
   if (lds > 64 * 1024) return -1;
   const int threads = o_dim >= 256 ? 256 : (o_dim + 63) / 64 * 64;
   dim3 grid((n + rows - 1) / rows, heads, (o_dim + threads - 1) / threads);
-#define QIL_HP(TX, TW, TO)                                                                                          \
-  hipLaunchKernelGGL((head_product_kernel<TX, TW, TO, 8>), grid, dim3(threads), lds, s, (const TX*)x, x_row, x_head, \
-                     (const TW*)w, (TO*)out, out_row, out_head, n, k_dim, o_dim)
+  const size_t w_bytes = w_dtype == QIL_F32 ? 4 : 2;
+  const bool few = n <= 32 && o_dim % 8 == 0 && (size_t)w % (8 * w_bytes) == 0 && lds + 4 * 8 * 64 * sizeof(float) <= 64 * 1024;
+  const dim3 grid_few((n + 7) / 8, heads, (o_dim + 63) / 64);
+#define QIL_HP(TX, TW, TO)                                                                                            \
+  do {                                                                                                                  \
+    if (few)                                                                                                            \
+      hipLaunchKernelGGL((head_product_few_kernel<TX, TW, TO>), grid_few, dim3(256), lds + 4 * 8 * 64 * sizeof(float), s, \
+                         (const TX*)x, x_row, x_head, (const TW*)w, (TO*)out, out_row, out_head, n, k_dim, o_dim);       \
+    else                                                                                                                \
+      hipLaunchKernelGGL((head_product_kernel<TX, TW, TO, 8>), grid, dim3(threads), lds, s, (const TX*)x, x_row, x_head, \
+                         (const TW*)w, (TO*)out, out_row, out_head, n, k_dim, o_dim);                                    \
+  } while (0)
   if (x_dtype == QIL_F32 && w_dtype == QIL_F32 && out_dtype == QIL_F32) QIL_HP(float, float, float);
   else if (x_dtype == QIL_BF16 && w_dtype == QIL_BF16 && out_dtype == QIL_F32) QIL_HP(bf16_t, bf16_t, float);
   else if (x_dtype == QIL_F32 && w_dtype == QIL_BF16 && out_dtype == QIL_BF16) QIL_HP(float, bf16_t, bf16_t);

@@ -295,7 +295,6 @@ int qil_latent_mfma(const float* q, const void* latent, const void* rope, const 
                                     cu_seqlens, seq_starts, n_seqs, single, parts == 1 ? sink : nullptr, out, part_acc, \
                                     part_m, part_l, heads, rank, rot, page_size, scale, rt, hb, P, parts)
   if (qf == 18 && vt == 32) QIL_LM(18, 32, true);
-  else if (qf == 5 && vt == 8) QIL_LM(5, 8, true);
   else if (qf <= 8 && vt <= 8) QIL_LM(8, 8, false);
   else if (qf <= 12 && vt <= 16) QIL_LM(12, 16, false);
   else QIL_LM(20, 32, false);
