@@ -98,28 +98,52 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
 #pragma unroll
   for (int t = 0; t < VT; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  const int chunks = dp / 8;
+  // Staging: a unit is two neighbouring keys by eight dims; a thread fetches up to NU units of the next step into
+  // registers while this step's products run.  The transposed copy takes a word per dim: the two keys' elements side
+  // by side, so that a wave's writes spread over the banks (a 2-byte write per key put 32 lanes on one bank).
+  constexpr int NU = (LM_KEYS / 2 * QF * 4 + LM_THREADS - 1) / LM_THREADS;
+  const int chunks = dp / 8, units = LM_KEYS / 2 * chunks;
+  uint4 ahead[NU][2];
+  auto fetch = [&](int j0) {
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+      const int idx = tid + LM_THREADS * u, jp = idx % (LM_KEYS / 2), dim = idx / (LM_KEYS / 2) * 8;
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int key = j0 + 2 * jp + e;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (idx < units && key < end && dim < d) {
+          const size_t slot = (size_t)table[key / page_size] * page_size + key % page_size;
+          v = dim < rank ? *reinterpret_cast<const uint4*>(latent + slot * rank + dim)
+                         : *reinterpret_cast<const uint4*>(rope + slot * rot + (dim - rank));
+        }
+        ahead[u][e] = v;
+      }
+    }
+  };
+  fetch(begin);
   for (int j0 = begin; j0 < end; j0 += LM_KEYS) {
     __syncthreads();                                        // the last step's reads are done
-    for (int idx = tid; idx < LM_KEYS * chunks; idx += LM_THREADS) {
-      const int j = idx / chunks, dim = (idx - j * chunks) * 8, key = j0 + j;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (key < end && dim < d) {
-        const size_t slot = (size_t)table[key / page_size] * page_size + key % page_size;
-        v = dim < rank ? *reinterpret_cast<const uint4*>(latent + slot * rank + dim)
-                       : *reinterpret_cast<const uint4*>(rope + slot * rot + (dim - rank));
-      }
-      *reinterpret_cast<uint4*>(ks + j * krow + dim) = v;
-      if (dim < rank) {
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          vts[(dim + 2 * e) * LM_VROW + j] = (bf16_t)(w[e] & 0xffffu);
-          vts[(dim + 2 * e + 1) * LM_VROW + j] = (bf16_t)(w[e] >> 16);
+    for (int u = 0; u < NU; ++u) {
+      const int idx = tid + LM_THREADS * u, jp = idx % (LM_KEYS / 2), dim = idx / (LM_KEYS / 2) * 8;
+      if (idx < units) {
+        const uint4 a = ahead[u][0], b = ahead[u][1];
+        *reinterpret_cast<uint4*>(ks + (2 * jp) * krow + dim) = a;
+        *reinterpret_cast<uint4*>(ks + (2 * jp + 1) * krow + dim) = b;
+        if (dim < rank) {
+          const uint32_t wa[4] = {a.x, a.y, a.z, a.w}, wb[4] = {b.x, b.y, b.z, b.w};
+          uint32_t* column = reinterpret_cast<uint32_t*>(vts) + jp;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            column[(dim + 2 * e) * (LM_VROW / 2)] = (wa[e] & 0xffffu) | (wb[e] << 16);
+            column[(dim + 2 * e + 1) * (LM_VROW / 2)] = (wa[e] >> 16) | (wb[e] & 0xffff0000u);
+          }
         }
       }
     }
     __syncthreads();
+    if (j0 + LM_KEYS < end) fetch(j0 + LM_KEYS);
     if (!working) continue;
     // ---- scores
     f32x4 sc[2];
