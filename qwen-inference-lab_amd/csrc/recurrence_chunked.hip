@@ -169,6 +169,7 @@ scan_carry_kernel(float* __restrict__ sums, float* __restrict__ norm_sums, const
   const size_t first = (size_t)block_place(row0, seq, 0) * heads + h;
   float top = MODE == QIL_SCAN_MLSTM ? carried[first] : 0.f;
   const double rate = MODE == QIL_SCAN_DECAY ? (double)decay[h] : 0.0;
+  const float keep_whole = MODE == QIL_SCAN_DECAY ? (float)pow(rate, (double)SCAN_BLOCK) : 0.f;   // a whole block's decay
   for (int c = 0; c < blocks; ++c) {
     const size_t at = first + (size_t)c * heads;
     float* u = e < mat ? sums + at * mat + e : norm_sums + at * dim + (e - mat);
@@ -180,7 +181,8 @@ scan_carry_kernel(float* __restrict__ sums, float* __restrict__ norm_sums, const
       if (e == 0) carried[at] = top;
       top = (float)(info[at * 2 + 1] + end);
     } else {
-      keep = (float)pow(rate, (double)min(SCAN_BLOCK, len - c * SCAN_BLOCK));
+      const int lc = min(SCAN_BLOCK, len - c * SCAN_BLOCK);
+      keep = lc == SCAN_BLOCK ? keep_whole : (float)pow(rate, (double)lc);
     }
     const float add = *u;
     *u = value;

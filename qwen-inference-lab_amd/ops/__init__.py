@@ -826,10 +826,15 @@ def latent_prepare(down, *, q_rank, rank, rot, q_weight, c_weight, eps, frequenc
     return out
 
 
+HEAD_PRODUCT_BLAS_ROWS = 256     # rows from which a bfloat16 product per head goes to the GPU BLAS in one batch
+
+
 def head_product(x, weight, *, heads, out_dtype, out=None, out_columns=None):
     """A product per head: x [N, heads * X] (head h's K inputs lead its X columns), weight [heads, K, O] (for every k
     its O outputs side by side) -> [N, heads * O] of ``out_dtype``, or into the leading O of every head's
-    ``out_columns`` columns of ``out``."""
+    ``out_columns`` columns of ``out``.  Own kernels for few rows (k split in a block) and in float32; bfloat16 weights
+    with ``HEAD_PRODUCT_BLAS_ROWS`` rows or more take one batched product of the GPU BLAS, float32 inputs rounded to
+    bfloat16 first."""
     n = x.shape[0]
     _require(x, 'x')
     _require(weight, 'weight')
@@ -840,6 +845,14 @@ def head_product(x, weight, *, heads, out_dtype, out=None, out_columns=None):
         out_columns = o
         out = torch.empty((n, heads * o), dtype=out_dtype, device=x.device)
     _require(out, 'out', out_dtype, (n, heads * out_columns))
+    if n >= HEAD_PRODUCT_BLAS_ROWS and weight.dtype == torch.bfloat16:
+        # many rows: one batched matrix-core product of the GPU BLAS (bfloat16 operands, float32 sums), a batch per head
+        inputs = x.view(n, heads, x.shape[1] // heads)[:, :, :k]
+        if inputs.dtype != torch.bfloat16:
+            inputs = inputs.to(torch.bfloat16)
+        product = torch.bmm(inputs.transpose(0, 1), weight)                    # [heads, N, O]
+        out.view(n, heads, out_columns)[:, :, :o].copy_(product.transpose(0, 1))
+        return out
     _check(library.load().qil_head_product(_ptr(x), _code(x.dtype), x.shape[1], x.shape[1] // heads, _ptr(weight),
                                            _code(weight.dtype), _ptr(out), _code(out_dtype), heads * out_columns,
                                            out_columns, n, heads, k, o, _stream()), 'head_product')

@@ -85,9 +85,9 @@ class MatrixMemory(Mixer):
         if self.position is not None:
             extra.update(frequencies=self.position.frequencies(), rot=self.rot)
         raw, below = ops.state_scan(proj, mode=self.gating, heads=self.heads, dim=self.dim, vdim=self.vdim, q_offset=0,
-                             k_offset=hd, v_offset=2 * hd, state=cache.state, cu_seqlens=ctx.cu_seqlens,
-                             seq_starts=ctx.seq_starts, seq_slots=ctx.seq_slots, n_seqs=ctx.n_seqs, q_scale=self.q_scale,
-                             k_scale=self.k_scale, max_query=ctx.max_query, **extra)
+                                    k_offset=hd, v_offset=2 * hd, state=cache.state, cu_seqlens=ctx.cu_seqlens,
+                                    seq_starts=ctx.seq_starts, seq_slots=ctx.seq_slots, n_seqs=ctx.n_seqs,
+                                    q_scale=self.q_scale, k_scale=self.k_scale, max_query=ctx.max_query, **extra)
         gated = ops.head_norm_gate(raw, proj, gate_offset=2 * hd + hv, heads=self.heads, vdim=self.vdim,
                                    weight=p.get('out_norm.weight'), eps=self.eps, gate=self.gate, out_dtype=self.dtype,
                                    denominators=below)

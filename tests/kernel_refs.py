@@ -240,8 +240,9 @@ def state_scan_slot(*, heads, dim, vdim, mode):
 
 
 def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, state, cu_seqlens, seq_starts, seq_slots,
-               n_seqs, gates=None, gate_bias=None, cap=0.0, decay=None, frequencies=None, rot=0, q_scale=1.0, k_scale=1.0):
-    """-> (o, denominators): for 'mlstm' o is undivided and the denominators are returned beside it.  The state slot's
+               n_seqs, gates=None, gate_bias=None, cap=0.0, decay=None, frequencies=None, rot=0, q_scale=1.0, k_scale=1.0,
+               max_query=None):
+    """Token by token whatever ``max_query`` says.  -> (o, denominators): for 'mlstm' o is undivided and the denominators are returned beside it.  The state slot's
     layout is the kernel's: matrices, then a normaliser per head, then the maximum tiles + 1 times per head."""
     n, tiles = proj.shape[0], -(-vdim // 16)
     x = proj.to(torch.float32)

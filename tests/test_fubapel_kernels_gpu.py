@@ -109,9 +109,11 @@ def test_latent_prepare_and_query(dtype):
 
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('sizes', [dict(n=3, heads=3, k=40, o=64), dict(n=9, heads=2, k=130, o=72), dict(n=32, heads=1, k=7, o=16),
-                                   dict(n=33, heads=2, k=40, o=64), dict(n=5, heads=4, k=33, o=20)])
+                                   dict(n=33, heads=2, k=40, o=64), dict(n=5, heads=4, k=33, o=20),
+                                   dict(n=300, heads=3, k=40, o=64), dict(n=257, heads=2, k=33, o=20)])
 def test_a_product_per_head_for_few_and_for_many_rows(dtype, sizes):
-    """Few rows with outputs in whole groups of eight take the kernel that splits k; other shapes the plain one."""
+    """Few rows with outputs in whole groups of eight take the kernel that splits k, many rows in bfloat16 the batched
+    product of the GPU BLAS, other shapes the plain kernel."""
     n, heads, k, o = sizes['n'], sizes['heads'], sizes['k'], sizes['o']
     g = torch.Generator().manual_seed(n * o)
     x = torch.randn(n, heads * k, generator=g)
