@@ -44,7 +44,7 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
   bf16_t* vts = ks + LM_KEYS * krow;                        // [rank][LM_VROW]: the latents, keys along a row
 
   // which rows: tile `tile` of rt rows of sequence s
-  int s = 0, tile = blockIdx.x;
+  int s = 0, tile = gridDim.x - 1 - blockIdx.x;             // the last tiles see the most keys: they start first
   if (single) {
     s = blockIdx.x;
     tile = 0;
@@ -77,13 +77,17 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
   bf16x8 qb[QF];
   {
     const float* qrow = q + gcol * d;
+    const bool wide = d % 4 == 0;                           // rows start on 16 bytes: two 16-byte reads a fragment
 #pragma unroll
     for (int f = 0; f < QF; ++f) {
       float x[8];
+      const int dim0 = 32 * f + 8 * kb;
+      if (wide && valid && f < qf && dim0 + 8 <= d) {
+        const float4 a = *reinterpret_cast<const float4*>(qrow + dim0), b = *reinterpret_cast<const float4*>(qrow + dim0 + 4);
+        x[0] = a.x, x[1] = a.y, x[2] = a.z, x[3] = a.w, x[4] = b.x, x[5] = b.y, x[6] = b.z, x[7] = b.w;
+      } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int dim = 32 * f + 8 * kb + e;
-        x[e] = (valid && f < qf && dim < d) ? qrow[dim] : 0.f;
+        for (int e = 0; e < 8; ++e) x[e] = (valid && f < qf && dim0 + e < d) ? qrow[dim0 + e] : 0.f;
       }
       qb[f] = __builtin_bit_cast(bf16x8, make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]),
                                                     pack_bf16(x[6], x[7])));
@@ -98,36 +102,47 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
 #pragma unroll
   for (int t = 0; t < VT; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  // Staging: a unit is two neighbouring keys by eight dims; a thread fetches up to NU units of the next step into
-  // registers while this step's products run.  The transposed copy takes a word per dim: the two keys' elements side
-  // by side, so that a wave's writes spread over the banks (a 2-byte write per key put 32 lanes on one bank).
-  constexpr int NU = (LM_KEYS / 2 * QF * 4 + LM_THREADS - 1) / LM_THREADS;
-  const int chunks = dp / 8, units = LM_KEYS / 2 * chunks;
+  // Staging: a unit is two neighbouring keys by eight dims; a thread owns one pair of keys (jp) and the chunks
+  // c0, c0 + 16, ... of their rows, and fetches its units of the next step into registers while this step's products
+  // run.  The keys' places in the cache (a table entry, a division) are found once a step and a step further ahead
+  // than the rows themselves, so that a row's read never waits for its table entry.  The transposed copy takes a word
+  // per dim: the two keys' elements side by side, so that a wave's writes spread over the banks (a 2-byte write per
+  // key put 32 lanes on one bank).
+  constexpr int CSTEP = LM_THREADS / (LM_KEYS / 2);
+  constexpr int NU = (QF * 4 + CSTEP - 1) / CSTEP;
+  const int chunks = dp / 8, jp = tid % (LM_KEYS / 2), c0 = tid / (LM_KEYS / 2);
   uint4 ahead[NU][2];
-  auto fetch = [&](int j0) {
+  int place[2];                                             // the cache slots of keys 2 jp, 2 jp + 1 of a step; -1: none
+  auto lookup = [&](int j0) {
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int key = j0 + 2 * jp + e;
+      place[e] = key < end ? table[key / page_size] * page_size + key % page_size : -1;
+    }
+  };
+  auto fetch = [&]() {
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
-      const int idx = tid + LM_THREADS * u, jp = idx % (LM_KEYS / 2), dim = idx / (LM_KEYS / 2) * 8;
+      const int chunk = c0 + CSTEP * u, dim = chunk * 8;
 #pragma unroll
       for (int e = 0; e < 2; ++e) {
-        const int key = j0 + 2 * jp + e;
         uint4 v = make_uint4(0, 0, 0, 0);
-        if (idx < units && key < end && dim < d) {
-          const size_t slot = (size_t)table[key / page_size] * page_size + key % page_size;
-          v = dim < rank ? *reinterpret_cast<const uint4*>(latent + slot * rank + dim)
-                         : *reinterpret_cast<const uint4*>(rope + slot * rot + (dim - rank));
-        }
+        if (chunk < chunks && place[e] >= 0 && dim < d)
+          v = dim < rank ? *reinterpret_cast<const uint4*>(latent + (size_t)place[e] * rank + dim)
+                         : *reinterpret_cast<const uint4*>(rope + (size_t)place[e] * rot + (dim - rank));
         ahead[u][e] = v;
       }
     }
   };
-  fetch(begin);
+  lookup(begin);
+  fetch();
+  lookup(begin + LM_KEYS);
   for (int j0 = begin; j0 < end; j0 += LM_KEYS) {
     __syncthreads();                                        // the last step's reads are done
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
-      const int idx = tid + LM_THREADS * u, jp = idx % (LM_KEYS / 2), dim = idx / (LM_KEYS / 2) * 8;
-      if (idx < units) {
+      const int chunk = c0 + CSTEP * u, dim = chunk * 8;
+      if (chunk < chunks) {
         const uint4 a = ahead[u][0], b = ahead[u][1];
         *reinterpret_cast<uint4*>(ks + (2 * jp) * krow + dim) = a;
         *reinterpret_cast<uint4*>(ks + (2 * jp + 1) * krow + dim) = b;
@@ -143,7 +158,10 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
       }
     }
     __syncthreads();
-    if (j0 + LM_KEYS < end) fetch(j0 + LM_KEYS);
+    if (j0 + LM_KEYS < end) {
+      fetch();
+      lookup(j0 + 2 * LM_KEYS);
+    }
     if (!working) continue;
     // ---- scores
     f32x4 sc[2];
@@ -185,11 +203,14 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
     // ---- U^T = U^T alpha + C^T P^T
     const bf16x8 pb = __builtin_bit_cast(bf16x8, make_uint4(pack_bf16(sc[0][0], sc[0][1]), pack_bf16(sc[0][2], sc[0][3]),
                                                             pack_bf16(sc[1][0], sc[1][1]), pack_bf16(sc[1][2], sc[1][3])));
+    const bool shrink = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;   // wave-uniform: some column's maximum rose
 #pragma unroll
     for (int t = 0; t < VT; ++t)
       if (EXACT || t < vt) {
+        if (shrink) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[t][i] *= alpha;
+          for (int i = 0; i < 4; ++i) o[t][i] *= alpha;
+        }
         o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(vts + (16 * t + r) * LM_VROW + 8 * kb),
                                                        pb, o[t], 0, 0, 0);
       }
