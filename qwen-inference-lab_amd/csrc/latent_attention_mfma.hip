@@ -13,7 +13,7 @@
 // keys 8 kb .. 8 kb + 7 and go into the second product's B operand as they are.  Scores, maxima, exponentials, sums
 // and results are float32; probabilities enter the second product as bfloat16.
 //
-// With few blocks the keys go in parts (grid.z): a block leaves (maximum, sum, unnormalised result) per column and
+// With few blocks the keys go in parts (grid.z): a block leaves (reference, sum, unnormalised result) per column and
 // part, and latent_merge_kernel finishes, which is also where the sink enters then.
 //
 // Takes rank % 16 == 0, rot % 8 == 0, rank + rot <= 640, rank <= 512; other sizes run on the general kernel.
@@ -26,6 +26,8 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define LM_KEYS 32
 #define LM_VROW (LM_KEYS + 8)                               // elements of a row of the transposed tile (80 bytes)
 #define LOG2E 1.44269504088896f
+#define LM_AHEAD 8                                          // LDS fragments asked for ahead of the product that takes them
+#define LM_SLACK 5.5f                                      // how far a score may pass the exponentials' reference
 
 // EXACT: the sizes are the template's (rank + rot == 32 QF up to padding, rank == 16 VT): no size guards the products.
 template <int QF, int VT, bool EXACT>
@@ -163,17 +165,27 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
       lookup(j0 + 2 * LM_KEYS);
     }
     if (!working) continue;
-    // ---- scores
-    f32x4 sc[2];
-#pragma unroll
-    for (int jt = 0; jt < 2; ++jt) {
-      const bf16_t* krow_p = ks + (8 * (r >> 2) + 4 * jt + (r & 3)) * krow + 8 * kb;
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    // ---- scores: the two sub-tiles' sums side by side; eight fragments of the staged keys are on their way from LDS
+    // before the first product, one more is asked for with every product
+    f32x4 sc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    {
+      const bf16_t* krow_p = ks + (8 * (r >> 2) + (r & 3)) * krow + 8 * kb;     // sub-tile 0; sub-tile 1 is four keys on
 #pragma unroll
       for (int f = 0; f < QF; ++f)
-        if (EXACT || f < qf)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(krow_p + 32 * f), qb[f], acc, 0, 0, 0);
-      sc[jt] = acc;
+        if (EXACT || f < qf) {
+          sc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(krow_p + 32 * f), qb[f], sc[0], 0, 0, 0);
+          sc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(krow_p + 4 * krow + 32 * f), qb[f],
+                                                          sc[1], 0, 0, 0);
+        }
+      if constexpr (EXACT) {
+        __builtin_amdgcn_sched_group_barrier(0x100, LM_AHEAD, 0);
+#pragma unroll
+        for (int i = 0; i < 2 * QF - LM_AHEAD; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, LM_AHEAD, 0);
+      }
     }
     float mx = -INFINITY;
 #pragma unroll
@@ -187,33 +199,50 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, QIL_WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, QIL_WAVE));
-    const float m_new = fmaxf(m, mx);
-    const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f((m - m_new) * LOG2E);
+    // The exponentials' reference m is a column's maximum as of some earlier step: it is raised, and the sums
+    // rescaled, only when a score passes it by more than LM_SLACK (so p <= exp(LM_SLACK), which float32 sums and
+    // bfloat16 probabilities hold as well as p <= 1).  In most steps no column of the wave rescales, and the
+    // accumulators stay where the matrix cores keep them.
+    const float m_new = (mx > m + LM_SLACK) ? mx : m;
+    if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {     // wave-uniform
+      asm volatile("" ::: "memory");                        // keeps this a branch: the multiplications are not speculated
+      const float alpha = (m_new == m) ? 1.f : __builtin_amdgcn_exp2f((m - m_new) * LOG2E);
+      l *= alpha;
+#pragma unroll
+      for (int t = 0; t < VT; ++t)
+        if (EXACT || t < vt) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[t][i] *= alpha;
+        }
+      m = m_new;
+    }
     float psum = 0.f;
 #pragma unroll
     for (int jt = 0; jt < 2; ++jt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = (sc[jt][i] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((sc[jt][i] - m_new) * LOG2E);
+        const float p = (sc[jt][i] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((sc[jt][i] - m) * LOG2E);
         sc[jt][i] = p;
         psum += p;
       }
-    l = l * alpha + psum;
-    m = m_new;
-    // ---- U^T = U^T alpha + C^T P^T
+    l += psum;
+    // ---- U^T += C^T P^T
     const bf16x8 pb = __builtin_bit_cast(bf16x8, make_uint4(pack_bf16(sc[0][0], sc[0][1]), pack_bf16(sc[0][2], sc[0][3]),
                                                             pack_bf16(sc[1][0], sc[1][1]), pack_bf16(sc[1][2], sc[1][3])));
-    const bool shrink = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;   // wave-uniform: some column's maximum rose
 #pragma unroll
     for (int t = 0; t < VT; ++t)
-      if (EXACT || t < vt) {
-        if (shrink) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) o[t][i] *= alpha;
-        }
+      if (EXACT || t < vt)
         o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(vts + (16 * t + r) * LM_VROW + 8 * kb),
                                                        pb, o[t], 0, 0, 0);
+    if constexpr (EXACT) {                                  // fragments ahead of the products, as for the scores
+      __builtin_amdgcn_sched_group_barrier(0x100, LM_AHEAD, 0);
+#pragma unroll
+      for (int i = 0; i < VT - LM_AHEAD; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
+      __builtin_amdgcn_sched_group_barrier(0x008, LM_AHEAD, 0);
+    }
   }
   if (!working) return;
   l += __shfl_xor(l, 16, QIL_WAVE);
