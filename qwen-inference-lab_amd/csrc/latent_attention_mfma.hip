@@ -268,30 +268,41 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
     if (EXACT || t < vt) *reinterpret_cast<float4*>(dst + 16 * t) = make_float4(o[t][0], o[t][1], o[t][2], o[t][3]);
 }
 
-// out[column] = sum_p w_p acc_p / (sum_p w_p l_p + exp(sink - M)), w_p = exp(m_p - M), M the largest of the parts' maxima
-// and the sink, over the parts that the row's position reaches.  One block per (row, head).
+// out[column] = sum_p w_p acc_p / (sum_p w_p l_p + exp(sink - M)), w_p = exp(m_p - M), M the largest of the parts'
+// references and the sink, over the parts that the row's position reaches.  One block per (row, head); the parts'
+// weights are made once, side by side, and kept in LDS (`parts` floats of dynamic LDS), so that the sums below wait
+// for no value that another read has to bring first.
 __global__ void latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_m,
                                     const float* __restrict__ part_l, const int* __restrict__ positions,
                                     const float* __restrict__ sink, float* __restrict__ out, int heads, int rank, int P,
                                     int parts) {
-  const int n = blockIdx.x, h = blockIdx.y;
+  extern __shared__ float weight[];
+  __shared__ float scratch[16];
+  const int n = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, nt = blockDim.x;
   const size_t column = (size_t)n * heads + h;
   const int reached = min(parts, positions[n] / P + 1);
   const float floor_ = sink ? sink[h] : -INFINITY;
   float top = floor_;
-  for (int p = 0; p < reached; ++p) top = fmaxf(top, part_m[column * parts + p]);
-  float below = sink ? expf(floor_ - top) : 0.f;
-  for (int p = 0; p < reached; ++p) {
+  for (int p = tid; p < reached; p += nt) {
     const float mp = part_m[column * parts + p];
-    if (mp > -INFINITY) below += expf(mp - top) * part_l[column * parts + p];
+    weight[p] = mp;
+    top = fmaxf(top, mp);
   }
-  for (int c = threadIdx.x; c < rank; c += blockDim.x) {
+  top = block_max(top, scratch);
+  float below = (sink && tid == 0) ? expf(floor_ - top) : 0.f;
+  for (int p = tid; p < reached; p += nt) {                 // a thread rereads only what it wrote
+    const float mp = weight[p], w = mp > -INFINITY ? expf(mp - top) : 0.f;
+    weight[p] = w;
+    below += w * part_l[column * parts + p];
+  }
+  below = block_sum(below, scratch);                        // its barriers also publish the weights
+  const float inv = 1.f / below;
+  const float* acc_p = part_acc + column * parts * rank;
+  for (int c = tid; c < rank; c += nt) {
     float acc = 0.f;
-    for (int p = 0; p < reached; ++p) {
-      const float mp = part_m[column * parts + p];
-      if (mp > -INFINITY) acc += expf(mp - top) * part_acc[(column * parts + p) * rank + c];
-    }
-    out[column * rank + c] = acc / below;
+#pragma unroll 4
+    for (int p = 0; p < reached; ++p) acc += weight[p] * acc_p[(size_t)p * rank + c];
+    out[column * rank + c] = acc * inv;
   }
 }
 
@@ -354,7 +365,7 @@ int qil_latent_mfma(const float* q, const void* latent, const void* rope, const 
                     float scale, int rt, int hb, int P, int parts, hipStream_t s) {
   if (n_rows == 0) return 0;
   if (!qil_latent_mfma_takes(heads, rank, rot) || page_size < 1 || rt < 1 || hb < 1 || rt * hb > 64 || P < 32 || P % 32 ||
-      parts < 1 || (single && n_seqs != n_rows) || (parts > 1 && !workspace))
+      parts < 1 || parts > 8192 || (single && n_seqs != n_rows) || (parts > 1 && !workspace))
     return -1;
   const int tiles = single ? n_seqs : (n_rows + rt - 1) / rt + n_seqs;
   dim3 grid(tiles, (heads + hb - 1) / hb, parts);
@@ -375,7 +386,7 @@ int qil_latent_mfma(const float* q, const void* latent, const void* rope, const 
 #undef QIL_LM
   if (status) return status;
   if (parts > 1)
-    hipLaunchKernelGGL(latent_merge_kernel, dim3(n_rows, heads), dim3(rank >= 256 ? 256 : 64), 0, s, part_acc, part_m,
+    hipLaunchKernelGGL(latent_merge_kernel, dim3(n_rows, heads), dim3(rank >= 256 ? 256 : 64), parts * sizeof(float), s, part_acc, part_m,
                        part_l, positions, sink, out, heads, rank, P, parts);
   QIL_RETURN_LAUNCH_STATUS();
 }
