@@ -22,27 +22,31 @@ template <typename TD, typename T>
 __global__ void latent_prepare_kernel(const TD* __restrict__ x, int splits, size_t split_stride, const float* __restrict__ wq,
                                       const float* __restrict__ wc, const float* __restrict__ freq,
                                       const int* __restrict__ positions, const int* __restrict__ slots, T* __restrict__ cq_out,
-                                      T* __restrict__ latent, T* __restrict__ rope, int q_rank, int rank, int rot, float eps) {
+                                      T* __restrict__ latent, T* __restrict__ rope, int q_rank, int rank, int rot, float eps, int held) {
+  extern __shared__ float sums[];                     // [q_rank + rank + rot] when `held`: the row, its partial sums added
   __shared__ float scratch[16];
   const int n = blockIdx.x, total = q_rank + rank + rot;
   const size_t at = (size_t)n * total;
+  if (held) {                                         // every element is read from memory once, all reads side by side
+    for (int i = threadIdx.x; i < total; i += blockDim.x) sums[i] = parts_sum(x, at + i, splits, split_stride);
+    __syncthreads();
+  }
+  auto value = [&](int i) { return held ? sums[i] : parts_sum(x, at + i, splits, split_stride); };
   float sq = 0.f, sc = 0.f;
-  for (int i = threadIdx.x; i < q_rank; i += blockDim.x) { const float v = parts_sum(x, at + i, splits, split_stride); sq += v * v; }
-  for (int i = threadIdx.x; i < rank; i += blockDim.x) { const float v = parts_sum(x, at + q_rank + i, splits, split_stride); sc += v * v; }
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x) { const float v = value(i); sq += v * v; }
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) { const float v = value(q_rank + i); sc += v * v; }
   sq = block_sum(sq, scratch);
   sc = block_sum(sc, scratch);
   const float rq = 1.f / sqrtf(sq / (float)q_rank + eps), rc = 1.f / sqrtf(sc / (float)rank + eps);
-  for (int i = threadIdx.x; i < q_rank; i += blockDim.x)
-    st(cq_out + (size_t)n * q_rank + i, parts_sum(x, at + i, splits, split_stride) * rq * wq[i]);
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x) st(cq_out + (size_t)n * q_rank + i, value(i) * rq * wq[i]);
   if (!slots) return;
   const size_t slot = (size_t)slots[n];
-  for (int i = threadIdx.x; i < rank; i += blockDim.x)
-    st(latent + slot * rank + i, parts_sum(x, at + q_rank + i, splits, split_stride) * rc * wc[i]);
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) st(latent + slot * rank + i, value(q_rank + i) * rc * wc[i]);
   const int half = rot / 2;
   const float p = (float)positions[n];
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
-    const float u = parts_sum(x, at + q_rank + rank + i, splits, split_stride);
-    const float v = parts_sum(x, at + q_rank + rank + half + i, splits, split_stride);
+    const float u = value(q_rank + rank + i);
+    const float v = value(q_rank + rank + half + i);
     float sn, cs;
     sincosf(p * freq[i], &sn, &cs);
     st(rope + slot * rot + i, u * cs - v * sn);
@@ -271,9 +275,11 @@ int qil_latent_prepare(const void* x, int x_dtype, int splits, const float* wq, 
   if (n == 0) return 0;
   if (q_rank < 1 || rank < 1 || rot < 2 || rot % 2 || splits < 1 || (x_dtype == QIL_BF16 && splits != 1)) return -1;
   const size_t stride = (size_t)n * (q_rank + rank + rot);
+  const size_t row_bytes = (size_t)(q_rank + rank + rot) * sizeof(float);
+  const int held = row_bytes <= 48 * 1024;            // the row's sums fit in LDS
 #define QIL_LP(TD, T)                                                                                               \
-  hipLaunchKernelGGL((latent_prepare_kernel<TD, T>), dim3(n), dim3(256), 0, s, (const TD*)x, splits, stride, wq, wc, \
-                     freq, positions, slots, (T*)cq_out, (T*)latent, (T*)rope, q_rank, rank, rot, eps)
+  hipLaunchKernelGGL((latent_prepare_kernel<TD, T>), dim3(n), dim3(256), held ? row_bytes : 0, s, (const TD*)x, splits, \
+                     stride, wq, wc, freq, positions, slots, (T*)cq_out, (T*)latent, (T*)rope, q_rank, rank, rot, eps, held)
   if (dtype == QIL_F32) {
     if (x_dtype != QIL_F32) return -1;
     QIL_LP(float, float);
