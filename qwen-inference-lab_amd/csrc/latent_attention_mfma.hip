@@ -30,8 +30,11 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define LM_SLACK 5.5f                                      // how far a score may pass the exponentials' reference
 
 // EXACT: the sizes are the template's (rank + rot == 32 QF up to padding, rank == 16 VT): no size guards the products.
-template <int QF, int VT, bool EXACT>
-__global__ void __launch_bounds__(LM_THREADS)
+// SPLIT (steps of single rows): the block's columns are at most 16, one wave's; every wave takes the scores of all of
+// them and a quarter of the latent's dims in the second product, so that four waves work where one would, each holds
+// a quarter of the sums, and two blocks fit a compute unit.
+template <int QF, int VT, bool EXACT, bool SPLIT>
+__global__ void __launch_bounds__(LM_THREADS, SPLIT ? 2 : 1)
 latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ latent, const bf16_t* __restrict__ rope,
                    const int* __restrict__ tables, int table_stride, const int* __restrict__ cu_seqlens,
                    const int* __restrict__ seq_starts, int n_seqs, int single, const float* __restrict__ sink,
@@ -69,9 +72,11 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, kb = lane >> 4;
-  const int column = wave * 16 + r, ci = column / hb, ch = column - ci * hb;
+  const int column = (SPLIT ? 0 : wave * 16) + r, ci = column / hb, ch = column - ci * hb;
   const bool valid = ci < rows_here && ch < heads_here && column < rt * hb;
-  const bool working = wave * 16 < rt * hb;                 // wave-uniform: this wave has columns at all
+  const bool working = SPLIT || wave * 16 < rt * hb;        // wave-uniform: this wave has columns at all
+  constexpr int VTW = SPLIT ? VT / 4 : VT;                  // tiles of 16 dims of the sums that this wave holds
+  const int t0 = SPLIT ? wave * VTW : 0;
   const int grow = seq_row0 + r0 + (valid ? ci : 0), head = h0 + (valid ? ch : 0);
   const int pos = valid ? start + r0 + ci : -1;
   const size_t gcol = (size_t)grow * heads + head;
@@ -100,9 +105,9 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
     m = sink[head];
     l = kb == 0 ? 1.f : 0.f;
   }
-  f32x4 o[VT];
+  f32x4 o[VTW];
 #pragma unroll
-  for (int t = 0; t < VT; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < VTW; ++t) o[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
   // Staging: a unit is two neighbouring keys by eight dims; a thread owns one pair of keys (jp) and the chunks
   // c0, c0 + 16, ... of their rows, and fetches its units of the next step into registers while this step's products
@@ -177,7 +182,7 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
           sc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(krow_p + 4 * krow + 32 * f), qb[f],
                                                           sc[1], 0, 0, 0);
         }
-      if constexpr (EXACT) {
+      if constexpr (EXACT && !SPLIT) {
         __builtin_amdgcn_sched_group_barrier(0x100, LM_AHEAD, 0);
 #pragma unroll
         for (int i = 0; i < 2 * QF - LM_AHEAD; ++i) {
@@ -209,8 +214,8 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
       const float alpha = (m_new == m) ? 1.f : __builtin_amdgcn_exp2f((m - m_new) * LOG2E);
       l *= alpha;
 #pragma unroll
-      for (int t = 0; t < VT; ++t)
-        if (EXACT || t < vt) {
+      for (int t = 0; t < VTW; ++t)
+        if (EXACT || t0 + t < vt) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) o[t][i] *= alpha;
         }
@@ -230,14 +235,14 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
     const bf16x8 pb = __builtin_bit_cast(bf16x8, make_uint4(pack_bf16(sc[0][0], sc[0][1]), pack_bf16(sc[0][2], sc[0][3]),
                                                             pack_bf16(sc[1][0], sc[1][1]), pack_bf16(sc[1][2], sc[1][3])));
 #pragma unroll
-    for (int t = 0; t < VT; ++t)
-      if (EXACT || t < vt)
-        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(vts + (16 * t + r) * LM_VROW + 8 * kb),
+    for (int t = 0; t < VTW; ++t)
+      if (EXACT || t0 + t < vt)
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(vts + (16 * (t0 + t) + r) * LM_VROW + 8 * kb),
                                                        pb, o[t], 0, 0, 0);
-    if constexpr (EXACT) {                                  // fragments ahead of the products, as for the scores
+    if constexpr (EXACT && !SPLIT) {                                  // fragments ahead of the products, as for the scores
       __builtin_amdgcn_sched_group_barrier(0x100, LM_AHEAD, 0);
 #pragma unroll
-      for (int i = 0; i < VT - LM_AHEAD; ++i) {
+      for (int i = 0; i < VTW - LM_AHEAD; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
@@ -250,22 +255,22 @@ latent_mfma_kernel(const float* __restrict__ q, const bf16_t* __restrict__ laten
   if (!valid) return;
   if (parts == 1) {
     const float inv = 1.f / l;
-    float* dst = out + gcol * rank + 4 * kb;
+    float* dst = out + gcol * rank + 16 * t0 + 4 * kb;
 #pragma unroll
-    for (int t = 0; t < VT; ++t)
-      if (EXACT || t < vt)
+    for (int t = 0; t < VTW; ++t)
+      if (EXACT || t0 + t < vt)
         *reinterpret_cast<float4*>(dst + 16 * t) = make_float4(o[t][0] * inv, o[t][1] * inv, o[t][2] * inv, o[t][3] * inv);
     return;
   }
   const size_t cell = gcol * parts + part;
-  if (kb == 0) {
+  if (kb == 0 && (!SPLIT || wave == 0)) {
     part_m[cell] = m;
     part_l[cell] = l;
   }
-  float* dst = part_acc + cell * rank + 4 * kb;
+  float* dst = part_acc + cell * rank + 16 * t0 + 4 * kb;
 #pragma unroll
-  for (int t = 0; t < VT; ++t)
-    if (EXACT || t < vt) *reinterpret_cast<float4*>(dst + 16 * t) = make_float4(o[t][0], o[t][1], o[t][2], o[t][3]);
+  for (int t = 0; t < VTW; ++t)
+    if (EXACT || t0 + t < vt) *reinterpret_cast<float4*>(dst + 16 * t) = make_float4(o[t][0], o[t][1], o[t][2], o[t][3]);
 }
 
 // out[column] = sum_p w_p acc_p / (sum_p w_p l_p + exp(sink - M)), w_p = exp(m_p - M), M the largest of the parts'
@@ -311,12 +316,12 @@ static int lm_lds_bytes(int rank, int rot) {
   return (LM_KEYS * (dp + 8) + rank * LM_VROW) * (int)sizeof(bf16_t);
 }
 
-template <int QF, int VT, bool EXACT>
+template <int QF, int VT, bool EXACT, bool SPLIT>
 static int lm_launch(dim3 grid, size_t lds, hipStream_t s, const float* q, const bf16_t* latent, const bf16_t* rope,
                      const int* tables, int table_stride, const int* cu_seqlens, const int* seq_starts, int n_seqs,
                      int single, const float* sink, float* out, float* part_acc, float* part_m, float* part_l, int heads,
                      int rank, int rot, int page_size, float scale, int rt, int hb, int P, int parts) {
-  auto kernel = latent_mfma_kernel<QF, VT, EXACT>;
+  auto kernel = latent_mfma_kernel<QF, VT, EXACT, SPLIT>;
   static bool raised = false;                                // per instantiation
   if (lds > 64 * 1024 && !raised) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -336,11 +341,12 @@ int qil_latent_mfma_takes(int heads, int rank, int rot) {
          lm_lds_bytes(rank, rot) <= 160 * 1024;
 }
 
-// (rows a block, heads a block, keys a part, parts) for a step: blocks of up to 64 columns; the keys in parts of at
-// least 128 while the blocks are fewer than two a compute unit.
+// (rows a block, heads a block, keys a part, parts) for a step: blocks of up to 64 columns (16 where every sequence
+// has one row: the split form); the keys in parts of at least 128 while the blocks are fewer than two a compute unit.
 void qil_latent_mfma_plan(int n_rows, int n_seqs, int single, int heads, int max_context, int* rt, int* hb, int* P,
                           int* parts) {
-  *hb = heads < 64 ? heads : 64;
+  const int most = single ? 16 : 64;                          // single rows: one wave's columns a block
+  *hb = heads < most ? heads : most;
   *rt = single ? 1 : (64 / *hb > 0 ? 64 / *hb : 1);
   const int tiles = single ? n_seqs : (n_rows + *rt - 1) / *rt + n_seqs;
   const long blocks = (long)tiles * ((heads + *hb - 1) / *hb);
@@ -364,7 +370,7 @@ int qil_latent_mfma(const float* q, const void* latent, const void* rope, const 
                     float* workspace, int n_rows, int n_seqs, int single, int heads, int rank, int rot, int page_size,
                     float scale, int rt, int hb, int P, int parts, hipStream_t s) {
   if (n_rows == 0) return 0;
-  if (!qil_latent_mfma_takes(heads, rank, rot) || page_size < 1 || rt < 1 || hb < 1 || rt * hb > 64 || P < 32 || P % 32 ||
+  if (!qil_latent_mfma_takes(heads, rank, rot) || page_size < 1 || rt < 1 || hb < 1 || rt * hb > (single ? 16 : 64) || P < 32 || P % 32 ||
       parts < 1 || parts > 8192 || (single && n_seqs != n_rows) || (parts > 1 && !workspace))
     return -1;
   const int tiles = single ? n_seqs : (n_rows + rt - 1) / rt + n_seqs;
@@ -375,15 +381,17 @@ int qil_latent_mfma(const float* q, const void* latent, const void* rope, const 
   float* part_l = parts > 1 ? part_m + (size_t)n_rows * heads * parts : nullptr;
   const int qf = (rank + rot + 31) / 32, vt = rank / 16;
   int status;
-#define QIL_LM(QF, VT, EXACT)                                                                                         \
-  status = lm_launch<QF, VT, EXACT>(grid, lds, s, q, (const bf16_t*)latent, (const bf16_t*)rope, tables, table_stride, \
-                                    cu_seqlens, seq_starts, n_seqs, single, parts == 1 ? sink : nullptr, out, part_acc, \
-                                    part_m, part_l, heads, rank, rot, page_size, scale, rt, hb, P, parts)
+#define QIL_LM_ARGS                                                                                                  \
+  grid, lds, s, q, (const bf16_t*)latent, (const bf16_t*)rope, tables, table_stride, cu_seqlens, seq_starts, n_seqs, \
+      single, parts == 1 ? sink : nullptr, out, part_acc, part_m, part_l, heads, rank, rot, page_size, scale, rt, hb, P, parts
+#define QIL_LM(QF, VT, EXACT) \
+  status = single ? lm_launch<QF, VT, EXACT, true>(QIL_LM_ARGS) : lm_launch<QF, VT, EXACT, false>(QIL_LM_ARGS)
   if (qf == 18 && vt == 32) QIL_LM(18, 32, true);
   else if (qf <= 8 && vt <= 8) QIL_LM(8, 8, false);
   else if (qf <= 12 && vt <= 16) QIL_LM(12, 16, false);
   else QIL_LM(20, 32, false);
 #undef QIL_LM
+#undef QIL_LM_ARGS
   if (status) return status;
   if (parts > 1)
     hipLaunchKernelGGL(latent_merge_kernel, dim3(n_rows, heads), dim3(rank >= 256 ? 256 : 64), parts * sizeof(float), s, part_acc, part_m,

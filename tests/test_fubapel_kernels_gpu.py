@@ -299,7 +299,8 @@ def test_head_norm_and_gate(dtype):
 
 
 @pytest.mark.parametrize('sizes', [dict(heads=5, rank=32, rot=8, page=4), dict(heads=6, rank=128, rot=32, page=16),
-                                   dict(heads=16, rank=512, rot=64, page=16), dict(heads=70, rank=48, rot=16, page=8)])
+                                   dict(heads=16, rank=512, rot=64, page=16), dict(heads=70, rank=48, rot=16, page=8),
+                                   dict(heads=40, rank=512, rot=64, page=32)])
 @pytest.mark.parametrize('step', ['portions', 'single rows', 'both'])
 @pytest.mark.parametrize('key_parts', [None, (64, 1), (32, 3)])
 def test_latent_attention_on_the_matrix_cores(sizes, step, key_parts, monkeypatch):
