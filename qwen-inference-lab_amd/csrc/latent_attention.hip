@@ -95,6 +95,7 @@ head_product_few_kernel(const TX* __restrict__ x, int x_row, int x_head, const T
   float* sums = xs + 8 * k_dim;
   const int row0 = blockIdx.x * 8, h = blockIdx.y, tid = threadIdx.x, to = tid & 7, kg = tid >> 3;
   const int o0 = blockIdx.z * 64 + to * 8;
+#pragma unroll 4
   for (int idx = tid; idx < 8 * k_dim; idx += 256) {
     const int r = idx / k_dim, k = idx - r * k_dim;
     xs[idx] = row0 + r < n_rows ? ld(x + (size_t)(row0 + r) * x_row + (size_t)h * x_head + k) : 0.f;
@@ -103,6 +104,7 @@ head_product_few_kernel(const TX* __restrict__ x, int x_row, int x_head, const T
   float acc[8][8] = {};
   if (o0 < o_dim) {
     const TW* wh = w + (size_t)h * k_dim * o_dim + o0;
+#pragma unroll 4                                      // four weight reads on their way at a time
     for (int k = kg; k < k_dim; k += 32) {
       float wv[8];
       ld8(wh + (size_t)k * o_dim, wv);

@@ -291,3 +291,27 @@ def test_the_plain_model_cuts_like_its_parts():
     whole, streams = plain.logits(tokens, weights, MIXED), []
     prefix = plain.logits(tokens[:17], weights, MIXED, streams=streams)
     assert torch.allclose(whole[:17], prefix, atol=1e-9) and len(streams) == 6 and plain.layer_order(MIXED) == [0, 1, 2, 1, 2, 3]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
+def test_trace_replay_program(tmp_path, dtype):
+    """``bin/trace_run`` on a Fubapel folder: requests alone and whole, their last tokens one by one, portions down to
+    two tokens, and up to four live requests in a pool of pages and state slots that is used again."""
+    from test_engine_gpu import collect, replay, traces
+    config, seed, _, spread = CONFIGS['mixed']
+    weights = plain.random_weights(config, seed, spread)
+    folder = write_model_folder(tmp_path / 'model', config, weights, torch.bfloat16)
+    prompts, shapes = traces(dict(vocab_size=config['vocab']), seed)
+    expected = {request: plain.logits(tokens, weights, config) for request, tokens in prompts.items()}
+    limit = LIMIT[getattr(torch, dtype)]
+    for shape, (steps, max_tokens) in shapes.items():
+        out = tmp_path / shape
+        replay(folder, dtype, steps, out, max_tokens)
+        rows = collect(out, steps, config['vocab'])
+        assert rows, shape
+        for request, items in rows.items():
+            got = torch.stack([row for _, row in items])
+            assert torch.isfinite(got).all()
+            e = error(got, expected[request][[position for position, _ in items]])
+            assert e <= limit, f'{shape} {request}: error {e:.3e}'
