@@ -298,7 +298,8 @@ def test_head_norm_and_gate(dtype):
                                        out_dtype=dtype, denominators=b), dtype, 3.0)
 
 
-@pytest.mark.parametrize('sizes', [dict(heads=5, rank=32, rot=8, page=4), dict(heads=6, rank=128, rot=32, page=16),
+@pytest.mark.parametrize('sizes', [dict(heads=5, rank=32, rot=8, page=4), dict(heads=7, rank=192, rot=40, page=16),
+                                   dict(heads=3, rank=400, rot=48, page=8),
                                    dict(heads=16, rank=512, rot=64, page=16), dict(heads=70, rank=48, rot=16, page=8),
                                    dict(heads=40, rank=512, rot=64, page=32)])
 @pytest.mark.parametrize('step', ['portions', 'single rows', 'both'])
