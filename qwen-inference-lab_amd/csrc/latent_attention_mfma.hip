@@ -342,7 +342,7 @@ int qil_latent_mfma_takes(int heads, int rank, int rot) {
 }
 
 // (rows a block, heads a block, keys a part, parts) for a step: blocks of up to 64 columns (16 where every sequence
-// has one row: the split form); the keys in parts of at least 128 while the blocks are fewer than two a compute unit.
+// has one row: the split form); the keys in parts of at least 64 while the blocks are fewer than two a compute unit.
 void qil_latent_mfma_plan(int n_rows, int n_seqs, int single, int heads, int max_context, int* rt, int* hb, int* P,
                           int* parts) {
   const int most = single ? 16 : 64;                          // single rows: one wave's columns a block
@@ -353,7 +353,7 @@ void qil_latent_mfma_plan(int n_rows, int n_seqs, int single, int heads, int max
   int want = (int)((2 * QIL_CUS + blocks - 1) / blocks);
   if (want < 1) want = 1;
   int part = ((max_context + want - 1) / want + 31) / 32 * 32;
-  if (part < 128) part = 128;
+  if (part < 64) part = 64;                                   // two steps a block: shorter parts cost more in the merge than they save
   *P = part;
   *parts = (max_context + part - 1) / part;
   if (*parts < 1) *parts = 1;
