@@ -2,5 +2,6 @@
 from .base import ConfigError, read_config_json
 from .qwen3 import Qwen3Config
 from .fubapel import FubapelConfig
+from .gerivik import GerivikConfig
 
-__all__ = ['ConfigError', 'read_config_json', 'Qwen3Config', 'FubapelConfig']
+__all__ = ['ConfigError', 'read_config_json', 'Qwen3Config', 'FubapelConfig', 'GerivikConfig']

@@ -66,7 +66,7 @@ attn_decode_kernel(FusedQKV fused, const bf16_t* __restrict__ q, int q_stride, c
                    const int* __restrict__ row_seq, const int* __restrict__ positions,
                    const int* __restrict__ row_index, float* __restrict__ part_acc, float* __restrict__ part_m,
                    float* __restrict__ part_l, bf16_t* __restrict__ out, int heads, int kv_heads, int d,
-                   int page_size, int window, float scale, int P, int parts) {
+                   int page_size, int window, float scale, int P, int parts, float softcap) {
   constexpr int QFRAGS = DMAX / 32, DTILES = DMAX / 16;
   if (WHOLE) d = DMAX;                                      // what the host has checked, known to the compiler: no
                                                             // condition on the head size stays in the loops
@@ -180,7 +180,9 @@ attn_decode_kernel(FusedQKV fused, const bf16_t* __restrict__ q, int q_stride, c
         const int key = k0 + 8 * kb + 4 * jt + i;
         const bool visible = key >= begin && key < end;
         keep[jt][i] = visible ? 0xffffu : 0u;
-        const float v = visible ? s[jt][i] * scale : -INFINITY;
+        float v = s[jt][i] * scale;
+        if (softcap > 0.f) v = soft_cap_fast(v, softcap, 2.88539008177793f / softcap);
+        if (!visible) v = -INFINITY;
         s[jt][i] = v;
         mx = fmaxf(mx, v);
       }
@@ -362,7 +364,7 @@ extern "C" int qil_attn_decode(const void* q, int q_stride, const void* k_cache,
                                const int* block_tables, int table_stride, const int* row_seq, const int* positions,
                                const int* row_index, void* workspace, void* out, int rows, int heads, int kv_heads,
                                int d, int page_size, int window, float scale, int P, int parts, int waves,
-                               int pairs, hipStream_t s) {
+                               int pairs, float softcap, hipStream_t s) {
   if (rows == 0) return 0;
   if (!qil_attn_decode_takes(heads, kv_heads, d, page_size) || P % 32 || P < 32 || parts < 1 || parts > 65535 ||
       kv_heads > 65535 || waves < 1 || waves > DEC_MAX_WAVES)
@@ -378,12 +380,12 @@ extern "C" int qil_attn_decode(const void* q, int q_stride, const void* k_cache,
   hipLaunchKernelGGL((attn_decode_kernel<DMAX, PAIRS, FUSED>), grid, dim3(waves * QIL_WAVE), lds, s, FIELDS,         \
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,       \
                      table_stride, row_seq, positions, row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d,        \
-                     page_size, window, scale, P, parts)
+                     page_size, window, scale, P, parts, softcap)
 #define QIL_DEC_WHOLE(DMAX, PAIRS)                                                                                  \
   hipLaunchKernelGGL((attn_decode_kernel<DMAX, PAIRS, false, true>), grid, dim3(waves * QIL_WAVE), lds, s, none,     \
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables,       \
                      table_stride, row_seq, positions, row_index, acc, m, l, (bf16_t*)out, heads, kv_heads, d,        \
-                     page_size, window, scale, P, parts)
+                     page_size, window, scale, P, parts, softcap)
 #define QIL_DEC_CASE(DMAX)                                                                                          \
   if (d == DMAX && pairs) QIL_DEC_WHOLE(DMAX, true);                                                                \
   else if (d == DMAX) QIL_DEC_WHOLE(DMAX, false);                                                                   \
@@ -417,6 +419,7 @@ extern "C" int qil_attn_decode_fused(const float* qkv, int splits, const float* 
                                      int heads, int kv_heads, int d, int page_size, int window, float scale, int P,
                                      int parts, int waves, int pairs, hipStream_t s) {
   if (rows == 0) return 0;
+  const float softcap = 0.f;                                 // (a capped attention makes its queries in qk_rope.hip)
   if (!qil_attn_decode_fused_takes(heads, kv_heads, d, page_size, cos_table ? rot : 0) || P % 32 || P < 32 ||
       parts < 1 || parts > 65535 || kv_heads > 65535 || waves < 1 || waves > DEC_MAX_WAVES || splits < 1 ||
       (q_weight == nullptr) != (k_weight == nullptr) || (cos_table == nullptr) != (sin_table == nullptr) ||

@@ -54,7 +54,7 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
                          const int* __restrict__ row_index, float* __restrict__ part_acc,
                          float* __restrict__ part_m, float* __restrict__ part_l,
                          T* __restrict__ out, int heads, int kv_heads, int d, int page_size, int window,
-                         float scale, int P, int parts, int tg_log2) {
+                         float scale, float softcap, int P, int parts, int tg_log2) {
   extern __shared__ float lds[];
   const int slot_row = blockIdx.x, kvh = blockIdx.y, part = blockIdx.z;   // slot_row indexes the workspace
   const int row = row_index ? row_index[slot_row] : slot_row;             // row of the step's batch
@@ -111,7 +111,7 @@ attn_rows_partial_kernel(const T* __restrict__ q, int q_stride, const T* __restr
 #pragma unroll
           for (int e = 0; e < 8; ++e) dot += qv[h][e] * kv[u][e];
           dot = group_sum(dot, tg_log2);
-          if (sub == 0 && t < count) scores[h * P + t] = dot * scale;
+          if (sub == 0 && t < count) scores[h * P + t] = soft_cap(dot * scale, softcap);
         }
       }
     }
@@ -300,7 +300,7 @@ static int launch_rows(const void* q, int q_stride, const void* k_cache, const v
                        int table_stride, const int* row_seq, const int* positions, const int* row_index,
                        float* part_acc, float* part_m,
                        float* part_l, void* out, int rows, int heads, int kv_heads, int d, int page_size, int window,
-                       float scale, int P, int parts, hipStream_t s, bool merge = true) {
+                       float scale, float softcap, int P, int parts, hipStream_t s, bool merge = true) {
   const int g = heads / kv_heads;
   const int gt = g >= 8 ? 8 : g > 2 ? 4 : g;            // head tile: 1, 2, 4 or 8
   const int tg_log2 = next_pow2_log2((d + 7) / 8);
@@ -309,7 +309,7 @@ static int launch_rows(const void* q, int q_stride, const void* k_cache, const v
 #define QIL_ROWS_CASE(GT)                                                                                          \
   hipLaunchKernelGGL((attn_rows_partial_kernel<T, GT>), grid, dim3(ATT_THREADS), lds, s, (const T*)q, q_stride,    \
                      (const T*)k_cache, (const T*)v_cache, block_tables, table_stride, row_seq, positions,         \
-                     row_index, part_acc, part_m, part_l, (T*)out, heads, kv_heads, d, page_size, window, scale, P, parts,    \
+                     row_index, part_acc, part_m, part_l, (T*)out, heads, kv_heads, d, page_size, window, scale, softcap, P, parts,    \
                      tg_log2)
   switch (gt) {
     case 1: QIL_ROWS_CASE(1); break;
@@ -342,7 +342,7 @@ size_t qil_attn_rows_workspace(int rows, int heads, int d, int parts) {
 int qil_attn_rows(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                   int table_stride, const int* row_seq, const int* positions, const int* row_index, void* workspace,
                   void* out, int rows,
-                  int heads, int kv_heads, int d, int page_size, int window, float scale, int P, int parts, int dtype,
+                  int heads, int kv_heads, int d, int page_size, int window, float scale, float softcap, int P, int parts, int dtype,
                   hipStream_t s) {
   if (rows == 0) return 0;
   if (d % 8 || d > 256 || d < 8 || heads % kv_heads || P < 1 || P > 1024 || parts < 1 || parts > 65535 ||
@@ -355,16 +355,16 @@ int qil_attn_rows(const void* q, int q_stride, const void* k_cache, const void* 
   float* l = m ? m + (size_t)rows * heads * parts : nullptr;
   if (dtype == QIL_F32)
     return launch_rows<float>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, row_index,
-                              acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s);
+                              acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, softcap, P, parts, s);
   return launch_rows<bf16_t>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, row_index,
-                             acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s);
+                             acc, m, l, out, rows, heads, kv_heads, d, page_size, window, scale, softcap, P, parts, s);
 }
 
 // The same without the merge: the parts' results stay in the workspace for a consumer that merges them itself
 // (parts > 1; `out` is not written).
 int qil_attn_rows_unmerged(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                            int table_stride, const int* row_seq, const int* positions, void* workspace, int rows,
-                           int heads, int kv_heads, int d, int page_size, int window, float scale, int P, int parts,
+                           int heads, int kv_heads, int d, int page_size, int window, float scale, float softcap, int P, int parts,
                            int dtype, hipStream_t s) {
   if (rows == 0) return 0;
   if (d % 8 || d > 256 || d < 8 || heads % kv_heads || P < 1 || P > 1024 || parts < 2 || parts > 65535 ||
@@ -377,9 +377,9 @@ int qil_attn_rows_unmerged(const void* q, int q_stride, const void* k_cache, con
   float* l = m + (size_t)rows * heads * parts;
   if (dtype == QIL_F32)
     return launch_rows<float>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, nullptr,
-                              acc, m, l, nullptr, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s, false);
+                              acc, m, l, nullptr, rows, heads, kv_heads, d, page_size, window, scale, softcap, P, parts, s, false);
   return launch_rows<bf16_t>(q, q_stride, k_cache, v_cache, block_tables, table_stride, row_seq, positions, nullptr,
-                             acc, m, l, nullptr, rows, heads, kv_heads, d, page_size, window, scale, P, parts, s, false);
+                             acc, m, l, nullptr, rows, heads, kv_heads, d, page_size, window, scale, softcap, P, parts, s, false);
 }
 
 // Merge of partial results written by a partial kernel (this file's or the matrix-core decode kernel's).

@@ -63,7 +63,11 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
                  const int* __restrict__ block_tables, int table_stride, const int* __restrict__ cu_seqlens,
                  const int* __restrict__ seq_starts, T* __restrict__ out, int heads, int kv_heads, int d,
                  int page_size, int window, float scale, int GH, int chunks, int ps_shift,
-                 float* __restrict__ part_acc, float* __restrict__ part_m, float* __restrict__ part_l, int P, int parts) {
+                 float* __restrict__ part_acc, float* __restrict__ part_m, float* __restrict__ part_l, int P, int parts,
+                 float softcap) {
+  // with a soft cap the scores are scaled and capped as they are made, and nothing is left for the exponent to scale
+  const float raw_scale = scale;
+  if (softcap > 0.f) scale = 1.f;
   using TT = TileTraits<T>;
   constexpr int BK = TT::BK, KSTEP = TT::KSTEP, PAD = TT::PAD;
   constexpr bool BF16 = sizeof(T) == 2;
@@ -337,6 +341,16 @@ attn_tile_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ k_
           }
       }
     }
+    if (softcap > 0.f) {
+      const float fast = 2.88539008177793f / softcap;
+#pragma unroll
+      for (int b = 0; b < RB; ++b)
+#pragma unroll
+        for (int jt = 0; jt < SUB; ++jt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            s[b][jt][i] = BF16 ? soft_cap_fast(s[b][jt][i] * raw_scale, softcap, fast) : soft_cap(s[b][jt][i] * raw_scale, softcap);
+    }
     // ---- mask and online softmax (per-lane row statistics).  m holds the running maximum of the RAW
     // scores; the scale (> 0) enters once, in the exponent: p = exp(scale * (s - m)).
     // every key of the tile is visible to every row of the wave unless the tile touches the wave's
@@ -472,7 +486,8 @@ template <typename T, int DMAX, int RB>
 static int launch_tile(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                        int table_stride, const int* cu_seqlens, const int* seq_starts, void* out, int n_seqs,
                        int max_query, int heads, int kv_heads, int d, int page_size, int window, float scale,
-                       hipStream_t s, float* workspace = nullptr, int total_rows = 0, int P = 0, int parts = 1) {
+                       hipStream_t s, float* workspace = nullptr, int total_rows = 0, int P = 0, int parts = 1,
+                       float softcap = 0.f) {
   using TT = TileTraits<T>;
   const int g = heads / kv_heads;
   const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = 4 / GH;
@@ -496,7 +511,7 @@ static int launch_tile(const void* q, int q_stride, const void* k_cache, const v
     if (page_size == (1 << b)) ps_shift = b;
   hipLaunchKernelGGL(kernel, grid, dim3(TILE_THREADS), lds, s, (const T*)q, q_stride, (const T*)k_cache,
                      (const T*)v_cache, block_tables, table_stride, cu_seqlens, seq_starts, (T*)out, heads, kv_heads, d,
-                     page_size, window, scale, GH, chunks, ps_shift, workspace, part_m, part_l, P, parts);
+                     page_size, window, scale, GH, chunks, ps_shift, workspace, part_m, part_l, P, parts, softcap);
   return (int)hipGetLastError();
 }
 
@@ -539,15 +554,15 @@ static int tile_dispatch(const void* q, int q_stride, const void* k_cache, const
                          const int* block_tables, int table_stride, const int* cu_seqlens, const int* seq_starts,
                          void* out, int n_seqs, int max_query, int heads, int kv_heads, int d, int page_size,
                          int window, float scale, int dtype, hipStream_t s, float* workspace, int total_rows, int P,
-                         int parts) {
+                         int parts, float softcap) {
   if (n_seqs == 0 || max_query < 2) return 0;
   if (d % 8 || d < 8 || d > 256 || heads % kv_heads || n_seqs > 65535 || kv_heads * 2 > 65535) return -1;
-  if (parts == 1 && dtype == QIL_BF16 && qil_attn_tile_bf16_takes(d, page_size, table_stride))
+  if (parts == 1 && softcap <= 0.f && dtype == QIL_BF16 && qil_attn_tile_bf16_takes(d, page_size, table_stride))
     return qil_attn_tile_bf16(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
                               n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s);
 #define QIL_TILE_CASE(T, DMAX)                                                                                      \
   return launch_tile<T, DMAX, (sizeof(T) == 2 && DMAX <= 128) ? 2 : 1>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, \
-                              n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s, workspace, total_rows, P, parts)
+                              n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s, workspace, total_rows, P, parts, softcap)
   if (dtype == QIL_F32) {
     if (d <= 64) QIL_TILE_CASE(float, 64);
     if (d <= 128) QIL_TILE_CASE(float, 128);
@@ -562,19 +577,19 @@ static int tile_dispatch(const void* q, int q_stride, const void* k_cache, const
 extern "C" int qil_attn_tile(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                              const int* block_tables, int table_stride, const int* cu_seqlens, const int* seq_starts,
                              void* out, int n_seqs, int max_query, int heads, int kv_heads, int d, int page_size,
-                             int window, float scale, int dtype, hipStream_t s) {
+                             int window, float scale, float softcap, int dtype, hipStream_t s) {
   return tile_dispatch(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, n_seqs,
-                       max_query, heads, kv_heads, d, page_size, window, scale, dtype, s, nullptr, 0, 0, 1);
+                       max_query, heads, kv_heads, d, page_size, window, scale, dtype, s, nullptr, 0, 0, 1, softcap);
 }
 
 extern "C" int qil_attn_tile_in_parts(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                       const int* block_tables, int table_stride, const int* cu_seqlens,
                                       const int* seq_starts, void* workspace, int total_rows, int n_seqs, int max_query,
-                                      int heads, int kv_heads, int d, int page_size, int window, float scale, int P,
-                                      int parts, int dtype, hipStream_t s) {
+                                      int heads, int kv_heads, int d, int page_size, int window, float scale,
+                                      float softcap, int P, int parts, int dtype, hipStream_t s) {
   if (n_seqs == 0 || max_query < 2) return 0;
   if (parts < 2 || P < 64 || P % 64 || !workspace || total_rows < 1) return -1;
   return tile_dispatch(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, nullptr, n_seqs,
                        max_query, heads, kv_heads, d, page_size, window, scale, dtype, s, (float*)workspace, total_rows,
-                       P, parts);
+                       P, parts, softcap);
 }

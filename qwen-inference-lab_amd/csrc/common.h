@@ -39,6 +39,14 @@ __device__ __forceinline__ float ld(const bf16_t* p) { return bf16_to_f32(*p); }
 __device__ __forceinline__ void st(float* p, float v) { *p = v; }
 __device__ __forceinline__ void st(bf16_t* p, float v) { *p = f32_to_bf16(v); }
 
+// A soft cap of attention scores: cap * tanh(score / cap); cap == 0 leaves the score as it is.  The second form
+// (the exponential and the reciprocal of the hardware, a few 1e-7 of the cap off) is for the bfloat16 kernels.
+__device__ __forceinline__ float soft_cap(float score, float cap) { return cap > 0.f ? cap * tanhf(score / cap) : score; }
+__device__ __forceinline__ float soft_cap_fast(float score, float cap, float doubled_log2e_over_cap) {
+  const float t = __builtin_amdgcn_exp2f(score * doubled_log2e_over_cap);       // exp(2 score / cap)
+  return cap - 2.f * cap * __builtin_amdgcn_rcpf(t + 1.f);                       // cap * (1 - 2 / (t + 1))
+}
+
 // Value after a round trip through T (what the reference's cast to the model dtype does).
 template <typename T> __device__ __forceinline__ float round_to(float v);
 template <> __device__ __forceinline__ float round_to<float>(float v) { return v; }

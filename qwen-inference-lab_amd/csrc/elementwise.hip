@@ -2,28 +2,30 @@
 // T is the model's element type (float or bfloat16); the residual stream is float32.
 #include "common.h"
 
-// stream[n, :] = float(table[token[n], :])                      (qil/model.py:126)
+// stream[n, :] = float(table[token[n], :]) * scale              (qil/model.py:126; scale 1 there)
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ tokens, const T* __restrict__ table,
-                             float* __restrict__ stream, int width) {
+                             float* __restrict__ stream, int width, float scale) {
   const int n = blockIdx.x;
   const T* row = table + (size_t)tokens[n] * width;
   float* out = stream + (size_t)n * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) out[i] = ld(row + i);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) out[i] = ld(row + i) * scale;
 }
 
 // The same for rows of bfloat16 whose width is a multiple of 8, 16-byte aligned: one thread, eight elements.
 __global__ void embed_bf16x8_kernel(const int* __restrict__ tokens, const bf16_t* __restrict__ table,
-                                    float* __restrict__ stream, int width) {
+                                    float* __restrict__ stream, int width, float scale) {
   const int n = blockIdx.x;
   const bf16_t* row = table + (size_t)tokens[n] * width;
   float* out = stream + (size_t)n * width;
   for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
     const uint4 raw = *reinterpret_cast<const uint4*>(row + i);
-    *reinterpret_cast<float4*>(out + i) = make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u),
-                                                      __uint_as_float(raw.y << 16), __uint_as_float(raw.y & 0xffff0000u));
-    *reinterpret_cast<float4*>(out + i + 4) = make_float4(__uint_as_float(raw.z << 16), __uint_as_float(raw.z & 0xffff0000u),
-                                                          __uint_as_float(raw.w << 16), __uint_as_float(raw.w & 0xffff0000u));
+    *reinterpret_cast<float4*>(out + i) =
+        make_float4(__uint_as_float(raw.x << 16) * scale, __uint_as_float(raw.x & 0xffff0000u) * scale,
+                    __uint_as_float(raw.y << 16) * scale, __uint_as_float(raw.y & 0xffff0000u) * scale);
+    *reinterpret_cast<float4*>(out + i + 4) =
+        make_float4(__uint_as_float(raw.z << 16) * scale, __uint_as_float(raw.z & 0xffff0000u) * scale,
+                    __uint_as_float(raw.w << 16) * scale, __uint_as_float(raw.w & 0xffff0000u) * scale);
   }
 }
 
@@ -206,16 +208,19 @@ __global__ void add_bias_kernel(T* __restrict__ x, const float* __restrict__ bia
 
 extern "C" {
 
-int qil_embed(const int* tokens, const void* table, float* stream, int n, int width, int dtype, hipStream_t s) {
+int qil_embed(const int* tokens, const void* table, float* stream, int n, int width, float scale, int dtype,
+              hipStream_t s) {
   if (n == 0) return 0;
   const int threads = width >= 1024 ? 256 : 64;
   if (dtype == QIL_F32)
-    hipLaunchKernelGGL(embed_kernel<float>, dim3(n), dim3(threads), 0, s, tokens, (const float*)table, stream, width);
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(n), dim3(threads), 0, s, tokens, (const float*)table, stream, width,
+                       scale);
   else if (width % 8 == 0 && (((uintptr_t)table | (uintptr_t)stream) % 16) == 0)
     hipLaunchKernelGGL(embed_bf16x8_kernel, dim3(n), dim3(width >= 2048 ? 256 : 64), 0, s, tokens, (const bf16_t*)table,
-                       stream, width);
+                       stream, width, scale);
   else
-    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(n), dim3(threads), 0, s, tokens, (const bf16_t*)table, stream, width);
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(n), dim3(threads), 0, s, tokens, (const bf16_t*)table, stream, width,
+                       scale);
   QIL_RETURN_LAUNCH_STATUS();
 }
 

@@ -1,0 +1,397 @@
+// A routed feed-forward (mixture of experts): the router, the grouping of (token, chosen expert) pairs by expert, the
+// experts' two products on the matrix cores, and the weighted sum.
+//
+//   route    per token: logits z = W_r h in float32 (W_r float32, h as it comes), scores s = softmax(z) over all
+//            outputs; choice scores c = s + correction; the outputs form `groups` equal groups of neighbours, a
+//            group's score is its largest c, and only the `keep` best groups stay (the others' c count as -inf);
+//            the `top` largest c are chosen (lowest index first among equals); the weights are their s, optionally
+//            divided by their sum.  The last `identity` outputs are experts without tensors that pass their input.
+//   align    pairs (token, slot) whose expert has tensors are put in the order of their experts, every expert's run
+//            cut into tiles of TM pairs: tile -> (expert, first place, pairs), a fixed number of tiles of which the
+//            unused ones hold no pair.  One block; the order inside an expert's run is whatever the atomics give,
+//            which no result depends on (every pair's row is a product of its own).
+//   gate_up  hidden[place] = act(W_gate,e h, W_up,e h) for the pairs of a tile, one wave per 16 hidden columns
+//   down     y[pair] = W_down,e hidden[place], float32
+//   combine  out[token] = sum over the token's slots, in slot order, of weight * (y[pair], or h for an identity expert)
+//
+// The products read their operands from memory in the matrix cores' own layout, 16 bytes a lane (a row's 8 bfloat16
+// or 4 float32 at k0 + 8 or 4 * (lane / 16)): v_mfma_f32_16x16x32_bf16, or four v_mfma_f32_16x16x4_f32 whose k runs
+// over the lanes' 4 elements in turn (true float32 products and sums).  A wave owns its output columns' weights, so a
+// block reads every weight once; the tile's rows of h are read by each wave again (from the caches).
+#include "common.h"
+#include "gated_act.h"
+
+typedef __bf16 moe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float moe_f32x4 __attribute__((ext_vector_type(4)));
+
+#define MOE_MAX_OUTPUTS 1024          // experts + identity experts the router takes
+#define MOE_ROUTE_THREADS 256
+
+// ------------------------------------------------------------------------------------------------ route
+__device__ __forceinline__ void wave_argmax(float& v, int& at) {          // the largest value, the lowest index among equals
+#pragma unroll
+  for (int o = QIL_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, QIL_WAVE);
+    const int oa = __shfl_xor(at, o, QIL_WAVE);
+    if (ov > v || (ov == v && oa < at)) { v = ov; at = oa; }
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(MOE_ROUTE_THREADS)
+moe_route_kernel(const T* __restrict__ x, int width, const float* __restrict__ w_router, const float* __restrict__ correction,
+                 int outputs, int groups, int keep, int top, int renormalize, int* __restrict__ chosen,
+                 float* __restrict__ weights) {
+  extern __shared__ float lds[];                        // [width] the row, [outputs] scores, [outputs] choice scores, [groups]
+  float* row = lds;
+  float* score = row + width;
+  float* choice = score + outputs;
+  float* group_best = choice + outputs;
+  const int n = blockIdx.x, lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) row[i] = ld(x + (size_t)n * width + i);
+  __syncthreads();
+  for (int e = wave; e < outputs; e += MOE_ROUTE_THREADS / QIL_WAVE) {
+    const float* w = w_router + (size_t)e * width;
+    float dot = 0.f;
+    for (int i = lane; i < width; i += QIL_WAVE) dot += row[i] * w[i];
+    dot = wave_sum(dot);
+    if (lane == 0) score[e] = dot;
+  }
+  __syncthreads();
+  // the rest is one wave's work; the others keep it company at the barriers between its steps
+  const bool mine = wave == 0;
+  if (mine) {
+    float top_logit = -INFINITY;
+    for (int e = lane; e < outputs; e += QIL_WAVE) top_logit = fmaxf(top_logit, score[e]);
+    top_logit = wave_max(top_logit);
+    float total = 0.f;
+    for (int e = lane; e < outputs; e += QIL_WAVE) total += expf(score[e] - top_logit);
+    total = wave_sum(total);
+    for (int e = lane; e < outputs; e += QIL_WAVE) {      // (a lane meets its own elements again)
+      const float s = expf(score[e] - top_logit) / total;
+      score[e] = s;
+      choice[e] = s + (correction ? correction[e] : 0.f);
+    }
+  }
+  __syncthreads();
+  if (groups > 1 && keep < groups) {
+    const int size = outputs / groups;
+    if (mine)
+      for (int g = lane; g < groups; g += QIL_WAVE) {
+        float best = -INFINITY;
+        for (int e = g * size; e < (g + 1) * size; ++e) best = fmaxf(best, choice[e]);
+        group_best[g] = best;
+      }
+    __syncthreads();
+    // the `keep` best groups are marked by +inf in their place, one after the other
+    for (int round = 0; round < keep; ++round) {
+      float v = -INFINITY;
+      int at = 0x7fffffff;
+      if (mine) {
+        for (int g = lane; g < groups; g += QIL_WAVE) {
+          const float gv = group_best[g];
+          if (gv != INFINITY && (gv > v || at == 0x7fffffff)) { v = gv; at = g; }
+        }
+        wave_argmax(v, at);
+      }
+      __syncthreads();
+      if (mine && lane == 0 && at != 0x7fffffff) group_best[at] = INFINITY;
+      __syncthreads();
+    }
+    if (mine)
+      for (int e = lane; e < outputs; e += QIL_WAVE)
+        if (group_best[e / size] != INFINITY) choice[e] = -INFINITY;
+    __syncthreads();
+  }
+  float sum = 0.f;
+  for (int round = 0; round < top; ++round) {
+    float v = -INFINITY;
+    int at = 0x7fffffff;
+    if (mine) {
+      for (int e = lane; e < outputs; e += QIL_WAVE) {
+        const float c = choice[e];
+        if (c == c && c != INFINITY && (c > v || at == 0x7fffffff)) { v = c; at = e; }   // +inf marks what is taken
+      }
+      wave_argmax(v, at);
+      if (at == 0x7fffffff) at = 0;
+      sum += score[at];
+    }
+    __syncthreads();
+    if (mine && lane == 0) {
+      chosen[(size_t)n * top + round] = at;
+      weights[(size_t)n * top + round] = score[at];
+      choice[at] = INFINITY;
+    }
+    __syncthreads();
+  }
+  if (renormalize && mine && lane < top) weights[(size_t)n * top + lane] = score[chosen[(size_t)n * top + lane]] / sum;
+}
+
+// ------------------------------------------------------------------------------------------------ align
+// tiles: [3][max_tiles] expert, first place, pairs.  places: [pairs] the pair at every place.
+__global__ void __launch_bounds__(1024)
+moe_align_kernel(const int* __restrict__ chosen, int pairs, int experts, int tile_rows, int max_tiles,
+                 int* __restrict__ tiles, int* __restrict__ places) {
+  __shared__ int count[MOE_MAX_OUTPUTS], first[MOE_MAX_OUTPUTS], first_tile[MOE_MAX_OUTPUTS + 1];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < experts; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int p = tid; p < pairs; p += blockDim.x) {
+    const int e = chosen[p];
+    if (e < experts) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int place = 0, tile = 0;
+    for (int e = 0; e < experts; ++e) {
+      first[e] = place;
+      first_tile[e] = tile;
+      place += count[e];
+      tile += (count[e] + tile_rows - 1) / tile_rows;
+    }
+    first_tile[experts] = tile;
+  }
+  __syncthreads();
+  for (int t = tid; t < max_tiles; t += blockDim.x) tiles[2 * max_tiles + t] = 0;
+  __syncthreads();
+  for (int e = tid; e < experts; e += blockDim.x) {
+    const int n_tiles = first_tile[e + 1] - first_tile[e];
+    for (int t = 0; t < n_tiles; ++t) {
+      const int at = first_tile[e] + t;
+      tiles[at] = e;
+      tiles[max_tiles + at] = first[e] + t * tile_rows;
+      tiles[2 * max_tiles + at] = min(tile_rows, count[e] - t * tile_rows);
+    }
+    count[e] = 0;                                       // from here on: the places of the expert's run already given out
+  }
+  __syncthreads();
+  for (int p = tid; p < pairs; p += blockDim.x) {
+    const int e = chosen[p];
+    if (e < experts) places[first[e] + atomicAdd(&count[e], 1)] = p;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ products
+template <typename T> struct Frag;
+template <> struct Frag<bf16_t> {
+  static constexpr int EPL = 8;                         // elements a lane holds of a row
+  typedef qil_u32x4 raw;
+  static __device__ __forceinline__ void mma(moe_f32x4& acc, const raw& a, const raw& b) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(moe_bf16x8, a), __builtin_bit_cast(moe_bf16x8, b), acc, 0, 0, 0);
+  }
+};
+template <> struct Frag<float> {
+  static constexpr int EPL = 4;
+  typedef moe_f32x4 raw;
+  static __device__ __forceinline__ void mma(moe_f32x4& acc, const raw& a, const raw& b) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], b[i], acc, 0, 0, 0);
+  }
+};
+
+// A lane's 16 bytes of a row at element k (zeros from `length` on; rows that are 16-byte aligned with a length that is
+// a multiple of EPL take one vector load, others go element by element).
+template <typename T, bool ALIGNED>
+__device__ __forceinline__ typename Frag<T>::raw load_frag(const T* __restrict__ row_ptr, int k, int length) {
+  typename Frag<T>::raw out;
+  if (ALIGNED) {
+    if (k < length) return *reinterpret_cast<const typename Frag<T>::raw*>(row_ptr + k);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = 0;
+    return out;
+  }
+  T e[Frag<T>::EPL];
+#pragma unroll
+  for (int i = 0; i < Frag<T>::EPL; ++i) e[i] = k + i < length ? row_ptr[k + i] : (T)0;
+  return __builtin_bit_cast(typename Frag<T>::raw, e);
+}
+
+// grid (tiles, ceil(ff / 64)); a wave: the tile's rows by 16 gate and the same 16 up columns.
+// w: [experts][2][ff][width] (an expert's gate rows, then its up rows).  hidden: [places][ff].
+template <typename T, int MT, bool ALIGNED>
+__global__ void __launch_bounds__(256)
+moe_gate_up_kernel(const T* __restrict__ x, int width, const T* __restrict__ w, int ff, const int* __restrict__ tiles,
+                   int max_tiles, const int* __restrict__ places, int top, T* __restrict__ hidden, int act, float limit,
+                   float alpha) {
+  constexpr int EPL = Frag<T>::EPL, KC = 4 * EPL;
+  const int tile = blockIdx.x, rows = tiles[2 * max_tiles + tile];
+  if (rows == 0) return;
+  const int e = tiles[tile], begin = tiles[max_tiles + tile];
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int col0 = (blockIdx.y * 4 + wave) * 16;
+  if (col0 >= ff) return;
+  const int r = lane & 15, kq = lane >> 4;
+  const T* a_row[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    const int local = m * 16 + r;
+    a_row[m] = x + (size_t)(places[begin + min(local, rows - 1)] / top) * width;
+  }
+  const int col = min(col0 + r, ff - 1);
+  const T* g_row = w + ((size_t)e * 2 * ff + col) * width;
+  const T* u_row = g_row + (size_t)ff * width;
+  moe_f32x4 acc_g[MT], acc_u[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) acc_g[m] = acc_u[m] = (moe_f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < width; k0 += KC) {
+    const int k = k0 + kq * EPL;
+    const typename Frag<T>::raw bg = load_frag<T, ALIGNED>(g_row, k, width), bu = load_frag<T, ALIGNED>(u_row, k, width);
+    typename Frag<T>::raw a[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) a[m] = load_frag<T, ALIGNED>(a_row[m], k, width);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      Frag<T>::mma(acc_g[m], a[m], bg);
+      Frag<T>::mma(acc_u[m], a[m], bu);
+    }
+  }
+  if (col0 + r >= ff) return;
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int local = m * 16 + 4 * kq + i;
+      if (local < rows) st(hidden + (size_t)(begin + local) * ff + col0 + r, gated_act(acc_g[m][i], acc_u[m][i], act, limit, alpha));
+    }
+}
+
+// grid (tiles, ceil(width / 128)); a wave: the tile's rows by 32 output columns.  w: [experts][width][ff].
+// y: [pairs][width] float32, a pair's row at the pair's own index.
+template <typename T, int MT, bool ALIGNED>
+__global__ void __launch_bounds__(256)
+moe_down_kernel(const T* __restrict__ hidden, int ff, const T* __restrict__ w, int width, const int* __restrict__ tiles,
+                int max_tiles, const int* __restrict__ places, float* __restrict__ y) {
+  constexpr int EPL = Frag<T>::EPL, KC = 4 * EPL;
+  const int tile = blockIdx.x, rows = tiles[2 * max_tiles + tile];
+  if (rows == 0) return;
+  const int e = tiles[tile], begin = tiles[max_tiles + tile];
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int col0 = (blockIdx.y * 4 + wave) * 32;
+  if (col0 >= width) return;
+  const int r = lane & 15, kq = lane >> 4;
+  const T* a_row[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) a_row[m] = hidden + (size_t)(begin + min(m * 16 + r, rows - 1)) * ff;
+  const T* b_row[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) b_row[t] = w + ((size_t)e * width + min(col0 + t * 16 + r, width - 1)) * ff;
+  moe_f32x4 acc[MT][2];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) acc[m][0] = acc[m][1] = (moe_f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < ff; k0 += KC) {
+    const int k = k0 + kq * EPL;
+    const typename Frag<T>::raw b0 = load_frag<T, ALIGNED>(b_row[0], k, ff), b1 = load_frag<T, ALIGNED>(b_row[1], k, ff);
+    typename Frag<T>::raw a[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) a[m] = load_frag<T, ALIGNED>(a_row[m], k, ff);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      Frag<T>::mma(acc[m][0], a[m], b0);
+      Frag<T>::mma(acc[m][1], a[m], b1);
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MT; ++m)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int local = m * 16 + 4 * kq + i;
+      if (local >= rows) continue;
+      float* out = y + (size_t)places[begin + local] * width;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+        if (col0 + t * 16 + r < width) out[col0 + t * 16 + r] = acc[m][t][i];
+    }
+}
+
+// out[n, c] = sum over slots, in slot order, of weight * (identity expert ? x[n, c] : y[n * top + slot, c])
+template <typename T>
+__global__ void moe_combine_kernel(const T* __restrict__ x, const float* __restrict__ y, const int* __restrict__ chosen,
+                                   const float* __restrict__ weights, int experts, int top, int width,
+                                   float* __restrict__ out) {
+  const int n = blockIdx.x;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float sum = 0.f;
+    for (int slot = 0; slot < top; ++slot) {
+      const size_t pair = (size_t)n * top + slot;
+      const float value = chosen[pair] >= experts ? ld(x + (size_t)n * width + c) : y[pair * width + c];
+      sum += weights[pair] * value;
+    }
+    out[(size_t)n * width + c] = sum;
+  }
+}
+
+extern "C" {
+
+int qil_moe_takes(int width, int outputs, int experts, int groups, int keep, int top) {
+  return width >= 1 && outputs >= 1 && outputs <= MOE_MAX_OUTPUTS && experts >= 0 && experts <= outputs && groups >= 1 &&
+         outputs % groups == 0 && keep >= 1 && keep <= groups && top >= 1 && top <= outputs && top <= QIL_WAVE &&
+         (size_t)(width + 2 * outputs + groups) * sizeof(float) <= 64 * 1024;
+}
+
+// x [n, width] (dtype), w_router float32 [outputs, width], correction float32 [outputs] or null -> chosen int32
+// [n, top], weights float32 [n, top].
+int qil_moe_route(const void* x, int dtype, const float* w_router, const float* correction, int* chosen, float* weights,
+                  int n, int width, int outputs, int groups, int keep, int top, int renormalize, hipStream_t s) {
+  if (n == 0) return 0;
+  if (!qil_moe_takes(width, outputs, 0, groups, keep, top)) return -1;
+  const size_t lds = (size_t)(width + 2 * outputs + groups) * sizeof(float);
+  if (dtype == QIL_F32)
+    hipLaunchKernelGGL(moe_route_kernel<float>, dim3(n), dim3(MOE_ROUTE_THREADS), lds, s, (const float*)x, width, w_router,
+                       correction, outputs, groups, keep, top, renormalize, chosen, weights);
+  else
+    hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(n), dim3(MOE_ROUTE_THREADS), lds, s, (const bf16_t*)x, width,
+                       w_router, correction, outputs, groups, keep, top, renormalize, chosen, weights);
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+// Rows a tile of pairs holds for a step of `pairs` pairs over `experts` experts: 16, or 64 when an expert's share
+// fills such tiles.
+int qil_moe_tile_rows(int pairs, int experts) { return experts > 0 && pairs / experts >= 48 ? 64 : 16; }
+int qil_moe_max_tiles(int pairs, int experts, int tile_rows) { return (pairs + tile_rows - 1) / tile_rows + experts; }
+
+// The experts' work on the routed pairs: x [n, width], chosen/weights [n, top]; w_gate_up [experts][2][ff][width],
+// w_down [experts][width][ff] (dtype); scratch: tiles int32 [3 * max_tiles], places int32 [n * top], hidden (dtype)
+// [n * top, ff], y float32 [n * top, width].  out float32 [n, width].
+int qil_moe_experts(const void* x, int dtype, const int* chosen, const float* weights, const void* w_gate_up,
+                    const void* w_down, int* tiles, int* places, void* hidden, float* y, float* out, int n, int width,
+                    int ff, int experts, int top, int tile_rows, int max_tiles, int act, float limit, float alpha,
+                    hipStream_t s) {
+  if (n == 0) return 0;
+  const int pairs = n * top;
+  if (experts > MOE_MAX_OUTPUTS || (tile_rows != 16 && tile_rows != 64) ||
+      max_tiles < qil_moe_max_tiles(pairs, experts, tile_rows) || width < 1 || ff < 1)
+    return -1;
+  if (experts > 0) {
+    hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), 0, s, chosen, pairs, experts, tile_rows, max_tiles, tiles,
+                       places);
+    const int epl = dtype == QIL_F32 ? 4 : 8;
+    const bool aligned = width % epl == 0 && ff % epl == 0 &&
+                         (((uintptr_t)x | (uintptr_t)w_gate_up | (uintptr_t)w_down | (uintptr_t)hidden) % 16) == 0;
+    const dim3 g_up(max_tiles, (ff + 63) / 64), g_down(max_tiles, (width + 127) / 128);
+#define QIL_MOE(T, MT, ALIGNED)                                                                                       \
+  do {                                                                                                                \
+    hipLaunchKernelGGL((moe_gate_up_kernel<T, MT, ALIGNED>), g_up, dim3(256), 0, s, (const T*)x, width,                \
+                       (const T*)w_gate_up, ff, tiles, max_tiles, places, top, (T*)hidden, act, limit, alpha);         \
+    hipLaunchKernelGGL((moe_down_kernel<T, MT, ALIGNED>), g_down, dim3(256), 0, s, (const T*)hidden, ff,               \
+                       (const T*)w_down, width, tiles, max_tiles, places, y);                                          \
+  } while (0)
+#define QIL_MOE_T(T)                                                                                                  \
+  do {                                                                                                                \
+    if (tile_rows == 64) { if (aligned) QIL_MOE(T, 4, true); else QIL_MOE(T, 4, false); }                              \
+    else { if (aligned) QIL_MOE(T, 1, true); else QIL_MOE(T, 1, false); }                                              \
+  } while (0)
+    if (dtype == QIL_F32) QIL_MOE_T(float); else QIL_MOE_T(bf16_t);
+#undef QIL_MOE_T
+#undef QIL_MOE
+  }
+  const int threads = width >= 1024 ? 256 : 64;
+  if (dtype == QIL_F32)
+    hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(n), dim3(threads), 0, s, (const float*)x, y, chosen, weights,
+                       experts, top, width, out);
+  else
+    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, dim3(n), dim3(threads), 0, s, (const bf16_t*)x, y, chosen, weights,
+                       experts, top, width, out);
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+}  // extern "C"

@@ -58,37 +58,54 @@ __device__ __forceinline__ void store8(bf16_t* p, const float* v) {
 // elements); every lane of the group must call.  x: the elements, replaced by the result (float32, to
 // be rounded to T when stored).  weight: null = no norm.  cos_table: null = no rotation; rot: rotated
 // width, pairs (i, i + rot / 2), rot / 16 a power of two.  d: the number of elements the norm's mean runs over.
+// sin_table null with a cos_table: the latter holds the rot / 2 frequencies, and the angle position * frequency,
+// its cosine and its sine are made here in float32 (no table bounds the positions).
+// rotate_first: the rotation comes before the norm (a design that norms what it has rotated).
 // (qil/model.py:15-23, 42-46, 52-55)
 template <typename T>
-__device__ __forceinline__ void norm_rope8(float (&x)[8], int chunk, int TG, const float* __restrict__ weight, int d,
-                                           float eps, const float* __restrict__ cos_table,
-                                           const float* __restrict__ sin_table, int position, int rot) {
-  if (weight) {
-    float sum = 0.f;
+__device__ __forceinline__ void head_norm8(float (&x)[8], int chunk, int TG, const float* __restrict__ weight, int d, float eps) {
+  float sum = 0.f;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) sum += x[e] * x[e];
-    for (int o = TG >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o, QIL_WAVE);
-    const float rstd = rsqrtf(sum / (float)d + eps);
-    const float4 w0 = *reinterpret_cast<const float4*>(weight + chunk * 8);
-    const float4 w1 = *reinterpret_cast<const float4*>(weight + chunk * 8 + 4);
-    const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+  for (int e = 0; e < 8; ++e) sum += x[e] * x[e];
+  for (int o = TG >> 1; o > 0; o >>= 1) sum += __shfl_xor(sum, o, QIL_WAVE);
+  const float rstd = rsqrtf(sum / (float)d + eps);
+  const float4 w0 = *reinterpret_cast<const float4*>(weight + chunk * 8);
+  const float4 w1 = *reinterpret_cast<const float4*>(weight + chunk * 8 + 4);
+  const float w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
 #pragma unroll
-    for (int e = 0; e < 8; ++e) x[e] = round_to<T>(x[e] * rstd) * w[e];
-  }
-  if (cos_table && rot > 0) {
-    const int half_chunks = rot >> 4;                   // chunks in half of the rotated width (a power of two)
-    float other[8];
+  for (int e = 0; e < 8; ++e) x[e] = round_to<T>(x[e] * rstd) * w[e];
+}
+__device__ __forceinline__ void rotate8(float (&x)[8], int chunk, const float* __restrict__ cos_table,
+                                        const float* __restrict__ sin_table, int position, int rot) {
+  const int half_chunks = rot >> 4;                   // chunks in half of the rotated width (a power of two)
+  float other[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) other[e] = __shfl_xor(x[e], half_chunks, QIL_WAVE);
-    if (chunk < 2 * half_chunks) {
-      const bool first = chunk < half_chunks;
+  for (int e = 0; e < 8; ++e) other[e] = __shfl_xor(x[e], half_chunks, QIL_WAVE);
+  if (chunk < 2 * half_chunks) {
+    const bool first = chunk < half_chunks;
+    float c[8], sn[8];
+    if (sin_table) {
       const size_t at = (size_t)position * (rot >> 1) + (first ? chunk : chunk - half_chunks) * 8;
       const float4 c0 = *reinterpret_cast<const float4*>(cos_table + at), c1 = *reinterpret_cast<const float4*>(cos_table + at + 4);
       const float4 s0 = *reinterpret_cast<const float4*>(sin_table + at), s1 = *reinterpret_cast<const float4*>(sin_table + at + 4);
-      const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-      const float sn[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+      c[0] = c0.x; c[1] = c0.y; c[2] = c0.z; c[3] = c0.w; c[4] = c1.x; c[5] = c1.y; c[6] = c1.z; c[7] = c1.w;
+      sn[0] = s0.x; sn[1] = s0.y; sn[2] = s0.z; sn[3] = s0.w; sn[4] = s1.x; sn[5] = s1.y; sn[6] = s1.z; sn[7] = s1.w;
+    } else {
+      const float* freq = cos_table + (first ? chunk : chunk - half_chunks) * 8;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) x[e] = first ? x[e] * c[e] - other[e] * sn[e] : other[e] * sn[e] + x[e] * c[e];
+      for (int e = 0; e < 8; ++e) sincosf((float)position * freq[e], &sn[e], &c[e]);
     }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = first ? x[e] * c[e] - other[e] * sn[e] : other[e] * sn[e] + x[e] * c[e];
   }
+}
+template <typename T>
+__device__ __forceinline__ void norm_rope8(float (&x)[8], int chunk, int TG, const float* __restrict__ weight, int d,
+                                           float eps, const float* __restrict__ cos_table,
+                                           const float* __restrict__ sin_table, int position, int rot,
+                                           bool rotate_first = false) {
+  const bool rotates = cos_table && rot > 0;
+  if (rotates && rotate_first) rotate8(x, chunk, cos_table, sin_table, position, rot);
+  if (weight) head_norm8<T>(x, chunk, TG, weight, d, eps);
+  if (rotates && !rotate_first) rotate8(x, chunk, cos_table, sin_table, position, rot);
 }

@@ -38,7 +38,7 @@ __global__ void qk_norm_rope_store_kernel(
     const float* __restrict__ q_weight, const float* __restrict__ k_weight,
     const float* __restrict__ cos_table, const float* __restrict__ sin_table, const int* __restrict__ positions,
     const int* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
-    int heads, int kv_heads, int d, int rot, int page_size, float eps, int norm_dim) {
+    int heads, int kv_heads, int d, int rot, int page_size, float eps, int norm_dim, int rotate_first) {
   __shared__ float vec[QIL_MAX_HEAD_DIM];
   const int n = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int total_heads = heads + 2 * kv_heads;
@@ -61,29 +61,46 @@ __global__ void qk_norm_rope_store_kernel(
   }
 
   const float* weight = is_q ? q_weight : k_weight;
-  float sum = 0.f;
-  for (int i = lane; i < d; i += QIL_WAVE) {
-    const float v = load_sum(qkv, src + i, splits, split_stride);
-    vec[i] = v;
-    sum += v * v;
+  for (int i = lane; i < d; i += QIL_WAVE) vec[i] = load_sum(qkv, src + i, splits, split_stride);
+  __syncthreads();
+  const int half = rot / 2;
+  const int position = positions[n];
+  const bool rotates = cos_table && rot > 0;
+  // one element of the rotated head: from the tables, or (no sine table) from the frequencies the cosine table's place holds
+  auto turned = [&](int i) {
+    if (!rotates || i >= rot) return vec[i];
+    const int f = i < half ? i : i - half;
+    float sn, cs;
+    if (sin_table) { cs = cos_table[(size_t)position * half + f]; sn = sin_table[(size_t)position * half + f]; }
+    else sincosf((float)position * cos_table[f], &sn, &cs);
+    return i < half ? vec[i] * cs - vec[i + half] * sn : vec[i - half] * sn + vec[i] * cs;
+  };
+  if (rotate_first) {                                    // rotate, then norm what was rotated
+    float mine[QIL_MAX_HEAD_DIM / QIL_WAVE], sum = 0.f;
+#pragma unroll
+    for (int u = 0; u < QIL_MAX_HEAD_DIM / QIL_WAVE; ++u) {
+      const int i = lane + u * QIL_WAVE;
+      mine[u] = i < d ? turned(i) : 0.f;
+      sum += mine[u] * mine[u];
+    }
+    float rstd = 1.f;
+    if (weight) rstd = rsqrtf(wave_sum(sum) / (float)norm_dim + eps);
+#pragma unroll
+    for (int u = 0; u < QIL_MAX_HEAD_DIM / QIL_WAVE; ++u) {
+      const int i = lane + u * QIL_WAVE;
+      if (i < d) st(dst + i, weight ? round_to<T>(mine[u] * rstd) * weight[i] : mine[u]);
+    }
+    return;
   }
   if (weight) {
+    float sum = 0.f;
+    for (int i = lane; i < d; i += QIL_WAVE) sum += vec[i] * vec[i];
     sum = wave_sum(sum);
     const float rstd = rsqrtf(sum / (float)norm_dim + eps);
     for (int i = lane; i < d; i += QIL_WAVE) vec[i] = round_to<T>(vec[i] * rstd) * weight[i];
+    __syncthreads();
   }
-  __syncthreads();
-  const int half = rot / 2;
-  const float* c = cos_table ? cos_table + (size_t)positions[n] * half : nullptr;
-  const float* s = sin_table ? sin_table + (size_t)positions[n] * half : nullptr;
-  for (int i = lane; i < d; i += QIL_WAVE) {
-    float v = vec[i];
-    if (c && i < rot) {
-      if (i < half) v = vec[i] * c[i] - vec[i + half] * s[i];
-      else          v = vec[i - half] * s[i - half] + vec[i] * c[i - half];
-    }
-    st(dst + i, v);
-  }
+  for (int i = lane; i < d; i += QIL_WAVE) st(dst + i, turned(i));
 }
 
 // The same work with eight consecutive elements a lane (16-byte vectors) and no LDS: a head is spread
@@ -98,7 +115,7 @@ qk_norm_rope_store_vec_kernel(
     const float* __restrict__ q_weight, const float* __restrict__ k_weight, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ slots,
     T* __restrict__ k_cache, T* __restrict__ v_cache, int n, int heads, int kv_heads, int d, int rot, int page_size,
-    float eps, int tg_log2, unsigned v_first_block, int norm_dim) {
+    float eps, int tg_log2, unsigned v_first_block, int norm_dim, int rotate_first) {
   const int total_heads = heads + 2 * kv_heads;
   const int TG = 1 << tg_log2;
   if (blockIdx.x >= v_first_block) {
@@ -140,7 +157,8 @@ qk_norm_rope_store_vec_kernel(
     for (int e = 0; e < 8; ++e) st(column + (size_t)e * page_size, x[e]);
     return;
   }
-  norm_rope8<T>(x, chunk, TG, is_q ? q_weight : k_weight, norm_dim, eps, cos_table, sin_table, positions[token], rot);
+  norm_rope8<T>(x, chunk, TG, is_q ? q_weight : k_weight, norm_dim, eps, cos_table, sin_table, positions[token], rot,
+                rotate_first != 0);
   if (is_q) {
     store8(q_out + ((size_t)token * heads + head) * d + chunk * 8, x);
   } else {
@@ -150,14 +168,16 @@ qk_norm_rope_store_vec_kernel(
   }
 }
 
+// sin_table null with a cos_table: cos_table holds the rot / 2 float32 frequencies and the kernels make the angle
+// position * frequency, its cosine and sine themselves.  rotate_first: rotate, then norm (else norm, then rotate).
 // qkv: in_dtype QIL_BF16 (one array, splits == 1) or QIL_F32 ([splits][n][..] partial sums).  dtype: type
 // of q_out and of the caches.  norm_dim: the number of elements the head norm's mean runs over (0: d); smaller
 // than d when the heads are padded with zeros to a size the attention kernels take.
 extern "C" int qil_qk_norm_rope_store(
     const void* qkv, int in_dtype, int splits, void* q_out, const float* q_weight, const float* k_weight,
     const float* cos_table, const float* sin_table, const int* positions, const int* slots, void* k_cache,
-    void* v_cache, int n, int heads, int kv_heads, int d, int rot, int page_size, float eps, int norm_dim, int dtype,
-    hipStream_t s) {
+    void* v_cache, int n, int heads, int kv_heads, int d, int rot, int page_size, float eps, int norm_dim, int rotate_first,
+    int dtype, hipStream_t s) {
   if (n == 0) return 0;
   if (norm_dim == 0) norm_dim = d;
   if (norm_dim < 1 || norm_dim > d) return -1;
@@ -184,7 +204,7 @@ extern "C" int qil_qk_norm_rope_store(
 #define QIL_QKV_CASE(TD, T)                                                                                           \
   hipLaunchKernelGGL((qk_norm_rope_store_vec_kernel<TD, T>), dim3(blocks), dim3(256), 0, s, (const TD*)qkv, splits,    \
                      stride, (T*)q_out, q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)k_cache,       \
-                     (T*)v_cache, n, heads, kv_heads, d, rot, page_size, eps, tg_log2, v_first_block, norm_dim)
+                     (T*)v_cache, n, heads, kv_heads, d, rot, page_size, eps, tg_log2, v_first_block, norm_dim, rotate_first)
     if (dtype == QIL_F32) QIL_QKV_CASE(float, float);
     else if (in_dtype == QIL_F32) QIL_QKV_CASE(float, bf16_t);
     else QIL_QKV_CASE(bf16_t, bf16_t);
@@ -194,7 +214,7 @@ extern "C" int qil_qk_norm_rope_store(
 #define QIL_QK_CASE(TD, T)                                                                                            \
   hipLaunchKernelGGL((qk_norm_rope_store_kernel<TD, T>), grid, dim3(QIL_WAVE), 0, s, (const TD*)qkv, splits, stride,   \
                      (T*)q_out, q_weight, k_weight, cos_table, sin_table, positions, slots, (T*)k_cache, (T*)v_cache,  \
-                     heads, kv_heads, d, rot, page_size, eps, norm_dim)
+                     heads, kv_heads, d, rot, page_size, eps, norm_dim, rotate_first)
   if (dtype == QIL_F32) QIL_QK_CASE(float, float);
   else if (in_dtype == QIL_F32) QIL_QK_CASE(float, bf16_t);
   else QIL_QK_CASE(bf16_t, bf16_t);

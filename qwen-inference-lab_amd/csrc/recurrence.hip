@@ -7,6 +7,9 @@
 //                   running maximum m_t = max(f_t + m_(t-1), i_t) with m = 0 before the first token,
 //                   a_t = exp(f_t + m_(t-1) - m_t), b_t = exp(i_t - m_t); a normaliser n_t = a_t n_(t-1) + b_t k_t;
 //                   o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6).
+//   QIL_SCAN_CHANNEL a decay of its own for every row of S (key channel i of head h) and token:
+//                   a_t[i] = sigmoid(z_t[h, i])^(1 / tau) = exp(logsigmoid(z_t[h, i]) / tau), b_t = 1, with z float32
+//                   [n, heads * dim] in the place of the gates and tau in the place of the cap; o_t as above.
 // Queries and keys may be rotated by position first (the leading rot elements of a head, element i with i + rot / 2,
 // angle position * freq[i]) and are then scaled (q_scale, k_scale).  Gates, rotation, state and sums are float32.
 //
@@ -24,7 +27,7 @@
 // position 0, and written back at the end.
 #include "common.h"
 
-enum { QIL_SCAN_DECAY = 0, QIL_SCAN_MLSTM = 1 };
+enum { QIL_SCAN_DECAY = 0, QIL_SCAN_MLSTM = 1, QIL_SCAN_CHANNEL = 2 };
 #define SCAN_CHUNK 16
 #define SCAN_COLUMNS 16                                          // state columns a block (one wave) owns
 
@@ -48,6 +51,7 @@ state_scan_kernel(const T* __restrict__ proj, int proj_row, int q_off, int k_off
   __shared__ __align__(16) float qs[CH][DMAX];
   __shared__ __align__(16) float ks[CH][DMAX];
   __shared__ float vs[CH][SCAN_COLUMNS];
+  __shared__ __align__(16) float as[MODE == QIL_SCAN_CHANNEL ? CH : 1][DMAX];    // CHANNEL: every row's decay, token by token
   __shared__ float fa[CH], fb[CH], fe[CH], gi[CH], gk[CH], gm[CH + 1];
   const int seq = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int tiles = (vdim + SCAN_COLUMNS - 1) / SCAN_COLUMNS;
@@ -80,7 +84,7 @@ state_scan_kernel(const T* __restrict__ proj, int proj_row, int q_off, int k_off
 
   // What a lane fetches of a chunk, all requests sent before any is used: elements lane + 64 u of the chunk's
   // [CH][DMAX] queries and keys, its own column of every token's values, and one token's gate inputs.
-  float rq[PER], rk[PER], rv[CH], rgi = 0.f, rgk = 0.f;
+  float rq[PER], rk[PER], rz[MODE == QIL_SCAN_CHANNEL ? PER : 1], rv[CH], rgi = 0.f, rgk = 0.f;
   auto fetch = [&](int c0) {
     const int cn = min(CH, row1 - c0);
 #pragma unroll
@@ -90,6 +94,7 @@ state_scan_kernel(const T* __restrict__ proj, int proj_row, int q_off, int k_off
       const T* x = proj + (size_t)(c0 + (live ? t : 0)) * proj_row + h * dim + (live ? i : 0);
       rq[u] = live ? ld(x + q_off) : 0.f;
       rk[u] = live ? ld(x + k_off) : 0.f;
+      if (MODE == QIL_SCAN_CHANNEL) rz[u] = live ? gates[(size_t)(c0 + t) * heads * dim + h * dim + i] : 0.f;
     }
 #pragma unroll
     for (int t = 0; t < CH; ++t)
@@ -109,6 +114,7 @@ state_scan_kernel(const T* __restrict__ proj, int proj_row, int q_off, int k_off
       const int idx = lane + 64 * u, t = idx / DMAX, i = idx % DMAX;
       qs[t][i] = i >= rot ? rq[u] * q_scale : rq[u];             // what is rotated is scaled behind the rotation
       ks[t][i] = i >= rot ? rk[u] * k_scale : rk[u];
+      if (MODE == QIL_SCAN_CHANNEL) as[t][i] = expf(log_sigmoid(rz[u]) / cap);
     }
     if (rg == 0) {
 #pragma unroll
@@ -159,10 +165,12 @@ state_scan_kernel(const T* __restrict__ proj, int proj_row, int q_off, int k_off
           if (4 * e < dim) {
             const float4 k4 = *reinterpret_cast<const float4*>(&ks[t][i]);
             const float4 q4 = *reinterpret_cast<const float4*>(&qs[t][i]);
-            col[e] = a * col[e] + k4.x * bv;         o += col[e] * q4.x;
-            col[e + 1] = a * col[e + 1] + k4.y * bv; o += col[e + 1] * q4.y;
-            col[e + 2] = a * col[e + 2] + k4.z * bv; o += col[e + 2] * q4.z;
-            col[e + 3] = a * col[e + 3] + k4.w * bv; o += col[e + 3] * q4.w;
+            float4 a4 = make_float4(a, a, a, a);
+            if (MODE == QIL_SCAN_CHANNEL) a4 = *reinterpret_cast<const float4*>(&as[t][i]);
+            col[e] = a4.x * col[e] + k4.x * bv;         o += col[e] * q4.x;
+            col[e + 1] = a4.y * col[e + 1] + k4.y * bv; o += col[e + 1] * q4.y;
+            col[e + 2] = a4.z * col[e + 2] + k4.z * bv; o += col[e + 2] * q4.z;
+            col[e + 3] = a4.w * col[e + 3] + k4.w * bv; o += col[e + 3] * q4.w;
           }
         }
         o += __shfl_xor(o, 16, QIL_WAVE);
@@ -241,6 +249,7 @@ int qil_state_scan_takes(int dim, int vdim, int rot) {
 
 // proj [n, proj_row] (dtype): a row holds the heads' queries from q_off, keys from k_off (heads x dim each) and
 // values from v_off (heads x vdim).  gates [n, 2 heads] float32 (inputs first, then keeps), gate_bias [2 heads]: MLSTM.
+// CHANNEL: gates [n, heads * dim] float32 (z, one per row of every head's state) and cap = tau.
 // decay [heads]: DECAY.  freq [rot / 2] or rot == 0.  out [n, heads * vdim] float32; MLSTM: undivided, with every
 // token's denominator in below [n, heads].
 int qil_state_scan(const void* proj, int dtype, int proj_row, int q_off, int k_off, int v_off, const float* gates,
@@ -248,8 +257,9 @@ int qil_state_scan(const void* proj, int dtype, int proj_row, int q_off, int k_o
                    float k_scale, float* state, const int* cu_seqlens, const int* seq_starts, const int* seq_slots,
                    float* out, float* below, int n_seqs, int heads, int dim, int vdim, int mode, hipStream_t s) {
   if (n_seqs == 0) return 0;
-  if (!qil_state_scan_takes(dim, vdim, rot) || (mode != QIL_SCAN_DECAY && mode != QIL_SCAN_MLSTM)) return -1;
-  if ((mode == QIL_SCAN_MLSTM && (!gates || !gate_bias || !below)) || (mode == QIL_SCAN_DECAY && !decay) || (rot && !freq)) return -1;
+  if (!qil_state_scan_takes(dim, vdim, rot) || mode < QIL_SCAN_DECAY || mode > QIL_SCAN_CHANNEL) return -1;
+  if ((mode == QIL_SCAN_MLSTM && (!gates || !gate_bias || !below)) || (mode == QIL_SCAN_DECAY && !decay) ||
+      (mode == QIL_SCAN_CHANNEL && (!gates || !(cap > 0.f))) || (rot && !freq)) return -1;
   const size_t slot_stride = qil_state_scan_slot(heads, dim, vdim, mode);
   dim3 grid(n_seqs, heads, (vdim + SCAN_COLUMNS - 1) / SCAN_COLUMNS + (mode == QIL_SCAN_MLSTM ? 1 : 0));
 #define QIL_SCAN(T, DMAX, MODE)                                                                                      \
@@ -264,9 +274,13 @@ int qil_state_scan(const void* proj, int dtype, int proj_row, int q_off, int k_o
     else QIL_SCAN(T, 256, MODE);                                                                                     \
   } while (0)
   if (dtype == QIL_F32) {
-    if (mode == QIL_SCAN_MLSTM) QIL_SCAN_DIM(float, QIL_SCAN_MLSTM); else QIL_SCAN_DIM(float, QIL_SCAN_DECAY);
+    if (mode == QIL_SCAN_MLSTM) QIL_SCAN_DIM(float, QIL_SCAN_MLSTM);
+    else if (mode == QIL_SCAN_CHANNEL) QIL_SCAN_DIM(float, QIL_SCAN_CHANNEL);
+    else QIL_SCAN_DIM(float, QIL_SCAN_DECAY);
   } else {
-    if (mode == QIL_SCAN_MLSTM) QIL_SCAN_DIM(bf16_t, QIL_SCAN_MLSTM); else QIL_SCAN_DIM(bf16_t, QIL_SCAN_DECAY);
+    if (mode == QIL_SCAN_MLSTM) QIL_SCAN_DIM(bf16_t, QIL_SCAN_MLSTM);
+    else if (mode == QIL_SCAN_CHANNEL) QIL_SCAN_DIM(bf16_t, QIL_SCAN_CHANNEL);
+    else QIL_SCAN_DIM(bf16_t, QIL_SCAN_DECAY);
   }
 #undef QIL_SCAN_DIM
 #undef QIL_SCAN

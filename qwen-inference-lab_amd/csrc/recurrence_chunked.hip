@@ -16,9 +16,16 @@
 //            S_in replaces its U, the last S_out goes to the state slot;
 //   outputs  per block: [q scaled by its carry weight | masked weighted q k^T] x [S_in ; v], tiled 64 tokens x 64 columns.
 // The tiled products run on the vector units in float32 (4 x 4 outputs a thread, operands staged in LDS).
+//
+// QIL_SCAN_CHANNEL (every row i of S decays by a factor of its own, a_t[i] = exp(logsigmoid(z_t[i]) / tau)): with
+// G_t[i] the sum of the block's log2 decays of row i up to token t (one more kernel, `decays`, walks them),
+//     S_t = diag(2^G_t) S_in + sum_(s <= t) diag(2^(G_t - G_s)) k_s v_s^T
+//     o_t = S_in^T (q_t * 2^G_t) + sum_(s <= t) (sum_i q_t[i] k_s[i] 2^(G_t[i] - G_s[i])) v_s
+// so `sums` weighs row i of k_s by 2^(G_end[i] - G_s[i]), `carry` keeps row i by 2^G_end[i], and `outputs` makes the
+// scores inside the block with the weight inside the sum over i (every exponent <= 0: nothing is divided by a decay).
 #include "common.h"
 
-enum { QIL_SCAN_DECAY = 0, QIL_SCAN_MLSTM = 1 };
+enum { QIL_SCAN_DECAY = 0, QIL_SCAN_MLSTM = 1, QIL_SCAN_CHANNEL = 2 };
 #define SCAN_BLOCK 64
 #define SCAN_TOP_TILE 16                                         // recurrence.hip keeps one maximum per 16 state columns
 
@@ -47,6 +54,29 @@ __device__ __forceinline__ GateLane gate_lane(const float* __restrict__ gates, c
 
 // Where block c of sequence seq keeps its sums: sequences before it took at most row0 / SCAN_BLOCK + seq places.
 __device__ __forceinline__ int block_place(int row0, int seq, int c) { return row0 / SCAN_BLOCK + seq + c; }
+
+// CHANNEL: gsum[row, e] = sum over the block's tokens up to this row of log2(a[e]), e over heads * dim; the sum runs
+// in float64 and is rounded once.  grid (blocks of the longest sequence, sequences, heads * dim / 256)
+__global__ void __launch_bounds__(256)
+scan_decays_kernel(const float* __restrict__ z, float tau, const int* __restrict__ cu_seqlens, float* __restrict__ gsum,
+                   int hd) {
+  const int c = blockIdx.x, seq = blockIdx.y, e = blockIdx.z * blockDim.x + threadIdx.x;
+  const int row0 = cu_seqlens[seq], len = cu_seqlens[seq + 1] - row0;
+  if (c * SCAN_BLOCK >= len || e >= hd) return;
+  const int r0 = row0 + c * SCAN_BLOCK, lc = min(SCAN_BLOCK, len - c * SCAN_BLOCK);
+  double sum = 0.0;
+  for (int t0 = 0; t0 < lc; t0 += 8) {
+    float in[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) in[u] = z[(size_t)(r0 + min(t0 + u, lc - 1)) * hd + e];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (t0 + u < lc) {
+        sum += (double)(log_sigmoid_c(in[u]) / tau) * 1.4426950408889634;
+        gsum[(size_t)(r0 + t0 + u) * hd + e] = (float)sum;
+      }
+  }
+}
 
 template <typename T>
 __global__ void scan_rotate_kernel(const T* __restrict__ proj, int proj_row, int q_off, int k_off,
@@ -79,7 +109,8 @@ scan_sums_kernel(const T* __restrict__ proj, int proj_row, int v_off, const floa
                  const float* __restrict__ decay, const float* __restrict__ state, size_t slot_stride,
                  const int* __restrict__ cu_seqlens, const int* __restrict__ seq_starts, const int* __restrict__ seq_slots,
                  float* __restrict__ sums, float* __restrict__ norm_sums, double* __restrict__ info,
-                 float* __restrict__ carried, int heads, int dim, int vdim, int dim_tiles) {
+                 float* __restrict__ carried, int heads, int dim, int vdim, int dim_tiles,
+                 const float* __restrict__ gsum) {
   __shared__ __align__(16) float kw[SCAN_BLOCK][64];
   __shared__ __align__(16) float vs[SCAN_BLOCK][64];
   __shared__ float w[SCAN_BLOCK];
@@ -109,6 +140,8 @@ scan_sums_kernel(const T* __restrict__ proj, int proj_row, int v_off, const floa
           carried[at] = seq_starts[seq] == 0 ? 0.f : *s_top;
         }
       }
+    } else if (MODE == QIL_SCAN_CHANNEL) {
+      weight = live ? 1.f : 0.f;                                 // (the rows' own weights follow below)
     } else {
       weight = live ? (float)pow((double)decay[h], (double)(lc - 1 - tid)) : 0.f;
     }
@@ -118,7 +151,11 @@ scan_sums_kernel(const T* __restrict__ proj, int proj_row, int v_off, const floa
   const size_t hd = (size_t)heads * dim;
   for (int idx = tid; idx < SCAN_BLOCK * 64; idx += 256) {
     const int s = idx / 64, x = idx % 64, i = it * 64 + x, j = jt * 64 + x;
-    kw[s][x] = (s < lc && i < dim) ? w[s] * qk[(size_t)(r0 + s) * 2 * hd + hd + (size_t)h * dim + i] : 0.f;
+    float weight = w[s];
+    if (MODE == QIL_SCAN_CHANNEL && s < lc && i < dim)
+      weight = __builtin_amdgcn_exp2f(gsum[(size_t)(r0 + lc - 1) * hd + (size_t)h * dim + i] -
+                                      gsum[(size_t)(r0 + s) * hd + (size_t)h * dim + i]);
+    kw[s][x] = (s < lc && i < dim) ? weight * qk[(size_t)(r0 + s) * 2 * hd + hd + (size_t)h * dim + i] : 0.f;
     vs[s][x] = (s < lc && j < vdim) ? ld(proj + (size_t)(r0 + s) * proj_row + v_off + h * vdim + j) : 0.f;
   }
   __syncthreads();
@@ -154,7 +191,7 @@ __global__ void __launch_bounds__(256)
 scan_carry_kernel(float* __restrict__ sums, float* __restrict__ norm_sums, const double* __restrict__ info,
                   float* __restrict__ carried, const float* __restrict__ decay, float* __restrict__ state,
                   size_t slot_stride, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_starts,
-                  const int* __restrict__ seq_slots, int heads, int dim, int vdim) {
+                  const int* __restrict__ seq_slots, int heads, int dim, int vdim, const float* __restrict__ gsum) {
   const int seq = blockIdx.x, h = blockIdx.y, e = blockIdx.z * blockDim.x + threadIdx.x;
   const int mat = dim * vdim, total = mat + (MODE == QIL_SCAN_MLSTM ? dim : 0);
   const int row0 = cu_seqlens[seq], len = cu_seqlens[seq + 1] - row0;
@@ -180,6 +217,9 @@ scan_carry_kernel(float* __restrict__ sums, float* __restrict__ norm_sums, const
       take = expf((float)(local - end));
       if (e == 0) carried[at] = top;
       top = (float)(info[at * 2 + 1] + end);
+    } else if (MODE == QIL_SCAN_CHANNEL) {
+      const int last = row0 + min((c + 1) * SCAN_BLOCK, len) - 1;       // the block's last token
+      keep = __builtin_amdgcn_exp2f(gsum[(size_t)last * heads * dim + (size_t)h * dim + e / vdim]);
     } else {
       const int lc = min(SCAN_BLOCK, len - c * SCAN_BLOCK);
       keep = lc == SCAN_BLOCK ? keep_whole : (float)pow(rate, (double)lc);
@@ -201,9 +241,12 @@ scan_outputs_kernel(const T* __restrict__ proj, int proj_row, int v_off, const f
                     const float* __restrict__ gates, const float* __restrict__ gate_bias, float cap,
                     const float* __restrict__ decay, const float* __restrict__ before, const float* __restrict__ norm_before,
                     const float* __restrict__ carried, const int* __restrict__ cu_seqlens, float* __restrict__ out,
-                    float* __restrict__ below, int heads, int dim, int vdim) {
-  // first the slabs [q^T | k^T | S_in rows], then [weighted scores^T | v]
-  __shared__ __align__(16) float stage[SCAN_BLOCK * OUT_PAD + SCAN_BLOCK * 64];
+                    float* __restrict__ below, int heads, int dim, int vdim, const float* __restrict__ gsum) {
+  // first the slabs [q^T | k^T | S_in rows] (CHANNEL: and [G^T | (q 2^G)^T]), then [weighted scores^T | v]
+  constexpr bool CHANNEL = MODE == QIL_SCAN_CHANNEL;
+  __shared__ __align__(16) float stage[SCAN_BLOCK * OUT_PAD + SCAN_BLOCK * 64 + (CHANNEL ? 2 * OUT_SLAB * OUT_PAD : 0)];
+  float* gT = stage + 2 * OUT_SLAB * OUT_PAD + OUT_SLAB * 64;
+  float* eT = gT + OUT_SLAB * OUT_PAD;
   __shared__ float nin[OUT_SLAB], cw[SCAN_BLOCK], em[SCAN_BLOCK], pw[SCAN_BLOCK + 1];
   __shared__ double lead[SCAN_BLOCK], tops[SCAN_BLOCK];
   float* qT = stage;
@@ -232,7 +275,7 @@ scan_outputs_kernel(const T* __restrict__ proj, int proj_row, int v_off, const f
       tops[tid] = top;
       cw[tid] = expf((float)(brought - top));
       em[tid] = expf(-(float)(g.sum + top));
-    } else {
+    } else if (!CHANNEL) {
       pw[tid] = (float)pow((double)decay[h], (double)tid);
       if (tid == 0) pw[SCAN_BLOCK] = (float)pow((double)decay[h], (double)SCAN_BLOCK);
     }
@@ -249,6 +292,11 @@ scan_outputs_kernel(const T* __restrict__ proj, int proj_row, int v_off, const f
       const float* src = qk + (size_t)(r0 + (ok ? t : 0)) * 2 * hd + (size_t)h * dim + (ok ? i : 0);
       qT[x * OUT_PAD + t] = ok ? src[0] : 0.f;
       kT[x * OUT_PAD + t] = ok ? src[hd] : 0.f;
+      if (CHANNEL) {
+        const float g = ok ? gsum[(size_t)(r0 + t) * hd + (size_t)h * dim + i] : 0.f;
+        gT[x * OUT_PAD + t] = g;
+        eT[x * OUT_PAD + t] = ok ? src[0] * __builtin_amdgcn_exp2f(g) : 0.f;
+      }
     }
     for (int idx = tid; idx < OUT_SLAB * 64; idx += 256) {
       const int x = idx / 64, y = idx % 64, i = i0 + x, j = jt * 64 + y;
@@ -263,6 +311,25 @@ scan_outputs_kernel(const T* __restrict__ proj, int proj_row, int v_off, const f
       const float4 s4 = *reinterpret_cast<const float4*>(&sin[x * 64 + tj * 4]);
       const float q[4] = {q4.x, q4.y, q4.z, q4.w}, k[4] = {k4.x, k4.y, k4.z, k4.w}, s[4] = {s4.x, s4.y, s4.z, s4.w};
       const float nx = MODE == QIL_SCAN_MLSTM ? nin[x] : 0.f;
+      if (CHANNEL) {
+        // the weight 2^(G_t - G_s) of every (query, key, row of S) inside the sum; what came in is taken by q 2^G_t
+        const float4 e4 = *reinterpret_cast<const float4*>(&eT[x * OUT_PAD + ti * 4]);
+        const float qe[4] = {e4.x, e4.y, e4.z, e4.w};
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) o[r][u] += qe[r] * s[u];
+        if (tj <= ti) {                                          // (tiles above the diagonal hold no visible key)
+          const float4 a4 = *reinterpret_cast<const float4*>(&gT[x * OUT_PAD + ti * 4]);
+          const float4 b4 = *reinterpret_cast<const float4*>(&gT[x * OUT_PAD + tj * 4]);
+          const float gt[4] = {a4.x, a4.y, a4.z, a4.w}, gs[4] = {b4.x, b4.y, b4.z, b4.w};
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) p[r][u] += q[r] * k[u] * __builtin_amdgcn_exp2f(fminf(gt[r] - gs[u], 0.f));
+        }
+        continue;
+      }
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
 #pragma unroll
@@ -278,13 +345,13 @@ scan_outputs_kernel(const T* __restrict__ proj, int proj_row, int v_off, const f
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int t = ti * 4 + r;
-    const float brought = MODE == QIL_SCAN_MLSTM ? cw[t] : pw[t + 1];
+    const float brought = MODE == QIL_SCAN_MLSTM ? cw[t] : CHANNEL ? 1.f : pw[t + 1];
     float row_sum = 0.f;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int s = tj * 4 + u;
       float weight = 0.f;
-      if (s <= t && t < lc) weight = MODE == QIL_SCAN_MLSTM ? expf((float)(lead[s] - tops[t])) : pw[t - s];
+      if (s <= t && t < lc) weight = MODE == QIL_SCAN_MLSTM ? expf((float)(lead[s] - tops[t])) : CHANNEL ? 1.f : pw[t - s];
       p[r][u] *= weight;
       row_sum += p[r][u];
       o[r][u] *= brought;
@@ -337,6 +404,7 @@ size_t qil_state_scan_chunked_workspace(int n, int n_seqs, int heads, int dim, i
   const size_t places = chunked_places(n, n_seqs);
   size_t floats = places * heads * 4 + (places * heads + 3) / 4 * 4 + (size_t)n * 2 * heads * dim + places * heads * dim * vdim;
   if (mode == QIL_SCAN_MLSTM) floats += places * heads * dim;
+  if (mode == QIL_SCAN_CHANNEL) floats += (size_t)n * heads * dim;
   return floats;
 }
 
@@ -348,15 +416,17 @@ int qil_state_scan_chunked(const void* proj, int dtype, int proj_row, int q_off,
                            int max_query, int heads, int dim, int vdim, int mode, hipStream_t s) {
   if (n_seqs == 0 || n == 0) return 0;
   if (dim < 1 || vdim < 1 || rot < 0 || rot % 2 || rot > dim || max_query < 1 ||
-      (mode != QIL_SCAN_DECAY && mode != QIL_SCAN_MLSTM) || !workspace || (size_t)n_seqs * heads > 65535)
+      mode < QIL_SCAN_DECAY || mode > QIL_SCAN_CHANNEL || !workspace || (size_t)n_seqs * heads > 65535)
     return -1;
-  if ((mode == QIL_SCAN_MLSTM && (!gates || !gate_bias || !below)) || (mode == QIL_SCAN_DECAY && !decay) || (rot && !freq)) return -1;
+  if ((mode == QIL_SCAN_MLSTM && (!gates || !gate_bias || !below)) || (mode == QIL_SCAN_DECAY && !decay) ||
+      (mode == QIL_SCAN_CHANNEL && (!gates || !(cap > 0.f) || n_seqs > 65535)) || (rot && !freq)) return -1;
   const size_t places = chunked_places(n, n_seqs);
   double* info = reinterpret_cast<double*>(workspace);
   float* carried = workspace + places * heads * 4;
   float* qk = carried + (places * heads + 3) / 4 * 4;
   float* sums = qk + (size_t)n * 2 * heads * dim;
   float* norm_sums = sums + places * heads * dim * vdim;
+  float* gsum = norm_sums;                                       // CHANNEL has no normaliser: its place holds the decays' sums
   const int blocks = (max_query + SCAN_BLOCK - 1) / SCAN_BLOCK;
   const int dim_tiles = (dim + 63) / 64, v_tiles = (vdim + 63) / 64;
   const int per_head = dim * vdim + (mode == QIL_SCAN_MLSTM ? dim : 0);
@@ -364,21 +434,28 @@ int qil_state_scan_chunked(const void* proj, int dtype, int proj_row, int q_off,
   const dim3 g_out(blocks, n_seqs * heads, v_tiles);
 #define QIL_CHUNKED(T, MODE)                                                                                          \
   do {                                                                                                                \
+    if (MODE == QIL_SCAN_CHANNEL)                                                                                     \
+      hipLaunchKernelGGL(scan_decays_kernel, dim3(blocks, n_seqs, (heads * dim + 255) / 256), dim3(256), 0, s, gates,  \
+                         cap, cu_seqlens, gsum, heads * dim);                                                          \
     hipLaunchKernelGGL(scan_rotate_kernel<T>, dim3(n), dim3(256), 0, s, (const T*)proj, proj_row, q_off, k_off, freq,  \
                        rot, q_scale, k_scale, cu_seqlens, seq_starts, n_seqs, qk, heads, dim);                         \
     hipLaunchKernelGGL((scan_sums_kernel<T, MODE>), g_sums, dim3(256), 0, s, (const T*)proj, proj_row, v_off, qk,      \
                        gates, gate_bias, cap, decay, state, slot_stride, cu_seqlens, seq_starts, seq_slots, sums,      \
-                       norm_sums, info, carried, heads, dim, vdim, dim_tiles);                                         \
+                       norm_sums, info, carried, heads, dim, vdim, dim_tiles, gsum);                                   \
     hipLaunchKernelGGL(scan_carry_kernel<MODE>, g_carry, dim3(256), 0, s, sums, norm_sums, info, carried, decay,       \
-                       state, slot_stride, cu_seqlens, seq_starts, seq_slots, heads, dim, vdim);                       \
+                       state, slot_stride, cu_seqlens, seq_starts, seq_slots, heads, dim, vdim, gsum);                 \
     hipLaunchKernelGGL((scan_outputs_kernel<T, MODE>), g_out, dim3(256), 0, s, (const T*)proj, proj_row, v_off, qk,    \
                        gates, gate_bias, cap, decay, sums, norm_sums, carried, cu_seqlens, out, below, heads, dim,     \
-                       vdim);                                                                                          \
+                       vdim, gsum);                                                                                    \
   } while (0)
   if (dtype == QIL_F32) {
-    if (mode == QIL_SCAN_MLSTM) QIL_CHUNKED(float, QIL_SCAN_MLSTM); else QIL_CHUNKED(float, QIL_SCAN_DECAY);
+    if (mode == QIL_SCAN_MLSTM) QIL_CHUNKED(float, QIL_SCAN_MLSTM);
+    else if (mode == QIL_SCAN_CHANNEL) QIL_CHUNKED(float, QIL_SCAN_CHANNEL);
+    else QIL_CHUNKED(float, QIL_SCAN_DECAY);
   } else {
-    if (mode == QIL_SCAN_MLSTM) QIL_CHUNKED(bf16_t, QIL_SCAN_MLSTM); else QIL_CHUNKED(bf16_t, QIL_SCAN_DECAY);
+    if (mode == QIL_SCAN_MLSTM) QIL_CHUNKED(bf16_t, QIL_SCAN_MLSTM);
+    else if (mode == QIL_SCAN_CHANNEL) QIL_CHUNKED(bf16_t, QIL_SCAN_CHANNEL);
+    else QIL_CHUNKED(bf16_t, QIL_SCAN_DECAY);
   }
 #undef QIL_CHUNKED
   QIL_RETURN_LAUNCH_STATUS();

@@ -152,6 +152,40 @@ class Normed:
         return add_rmsnorm(self.stream, None, self.weight, self.eps, self.dtype)
 
 
+class PostNormed:
+    """A sub-layer output that joins the residual stream as its RMS norm: stream += value / rms(value) * weight.
+    ``value``: tensor of the model's type, float32 tensor, or ``Partials``.  The norms that add a pending output
+    (``add_rmsnorm``, ``rows_rmsnorm``) take it and make both norms in one kernel, in float32 throughout."""
+
+    def __init__(self, value, weight, eps):
+        self.value, self.weight, self.eps = value, weight, float(eps)
+        self.shape, self.device = tuple(value.shape), value.device
+
+
+def _post_normed(stream, pending, rows, weight, eps, out_dtype, update):
+    n, width = stream.shape
+    value = pending.value
+    _require(stream, 'stream', torch.float32)
+    _require(weight, 'weight', torch.float32, (width,))
+    _require(pending.weight, 'post-norm weight', torch.float32, (width,))
+    if isinstance(value, Partials):
+        _require(value.tensor, 'delta', torch.float32, (value.splits, n, width))
+        pointer, code, splits = value.tensor.data_ptr(), 0, value.splits
+    else:
+        _require(value, 'delta', None, (n, width))
+        if value.dtype not in (torch.float32, out_dtype):
+            raise ValueError(f'delta must be float32 or {out_dtype}')
+        pointer, code, splits = value.data_ptr(), _code(value.dtype), 1
+    if rows is not None:
+        _require(rows, 'rows', torch.int32)
+    count = n if rows is None else rows.shape[0]
+    out = torch.empty((count, width), dtype=out_dtype, device=stream.device)
+    _check(library.load().qil_post_norm_add_norm(_ptr(stream), pointer, code, splits, n, _ptr(pending.weight), pending.eps,
+                                                 _ptr(rows), _ptr(weight), _ptr(out), count, width, float(eps),
+                                                 int(update), _code(out_dtype), _stream()), 'post_norm_add_norm')
+    return out
+
+
 def _operand(value, name, model_dtype, shape):
     """(pointer, dtype code, splits) of a consumer's input: a tensor of the model's type or Partials."""
     if isinstance(value, Partials):
@@ -224,14 +258,14 @@ def _check_caches(k_cache, v_cache, dtype, kv_heads, page_size, head_dim):
         raise ValueError(f'v_cache must be [pages, {kv_heads}, {head_dim}, {page_size}]')
 
 
-def embed(token_ids, table):
-    """int32 [N], T [V, H] -> float32 stream [N, H]."""
+def embed(token_ids, table, scale=1.0):
+    """int32 [N], T [V, H] -> float32 stream [N, H] = table[token] * scale."""
     library.check_device()                                 # every step begins here
     _require(token_ids, 'token_ids', torch.int32)
     _require(table, 'table')
     n, width = token_ids.shape[0], table.shape[1]
     stream = torch.empty((n, width), dtype=torch.float32, device=table.device)
-    _check(library.load().qil_embed(_ptr(token_ids), _ptr(table), _ptr(stream), n, width, _code(table.dtype),
+    _check(library.load().qil_embed(_ptr(token_ids), _ptr(table), _ptr(stream), n, width, float(scale), _code(table.dtype),
                                     _stream()), 'embed')
     return stream
 
@@ -239,7 +273,9 @@ def embed(token_ids, table):
 def add_rmsnorm(stream, delta, weight, eps, out_dtype):
     """stream += delta (in place, float32 sum; skipped if delta is None); returns norm(stream) as out_dtype.
 
-    ``delta``: tensor of ``out_dtype`` [N, H] or Partials."""
+    ``delta``: tensor of ``out_dtype`` [N, H], Partials, or a ``PostNormed`` (its norm is what is added)."""
+    if isinstance(delta, PostNormed):
+        return _post_normed(stream, delta, None, weight, eps, out_dtype, True)
     n, width = stream.shape
     _require(stream, 'stream', torch.float32)
     _require(weight, 'weight', torch.float32, (width,))
@@ -252,6 +288,8 @@ def add_rmsnorm(stream, delta, weight, eps, out_dtype):
 
 def rows_rmsnorm(stream, delta, rows, weight, eps, out_dtype):
     """norm(stream[rows] + delta[rows]) as out_dtype [len(rows), H]; stream is left as it is."""
+    if isinstance(delta, PostNormed):
+        return _post_normed(stream, delta, rows, weight, eps, out_dtype, False)
     n, width = stream.shape
     _require(stream, 'stream', torch.float32)
     _require(weight, 'weight', torch.float32, (width,))
@@ -469,10 +507,32 @@ def silu_mul(gate_up, out_dtype=None, interleaved=False):
     return out
 
 
+def _rotation_arguments(rotation, head_dim):
+    """(cos or frequencies, sin or None, rotated width) of a ``Rotation`` for the kernels: tables [positions, rot / 2],
+    or (``rotation.frequencies``) the rot / 2 float32 frequencies alone, from which the kernels make the angles."""
+    if rotation is None:
+        return None, None, 0
+    rot = rotation.rot_dim
+    if getattr(rotation, 'frequencies', None) is not None:
+        _require(rotation.frequencies, 'frequencies', torch.float32, (rot // 2,))
+        cos, sin = rotation.frequencies, None
+    else:
+        cos, sin = rotation.cos, rotation.sin
+        _require(cos, 'cos', torch.float32)
+        _require(sin, 'sin', torch.float32, cos.shape)
+        if cos.shape[1] * 2 != rot:
+            raise ValueError('rotation tables do not fit rot_dim')
+    if rot > head_dim or rot % 2:
+        raise ValueError('rotation does not fit the head')
+    return cos, sin, rot
+
+
 def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, slots,
-                       k_cache, v_cache, page_size, dtype, norm_dim=None):
+                       k_cache, v_cache, page_size, dtype, norm_dim=None, rotate_first=False):
     """Per-head RMSNorm of q and k (if weights are given), rotation by position (if given).  ``norm_dim``: the
     number of elements the norm's mean runs over when the heads are padded with zeros (default: head_dim).
+    ``rotate_first``: the rotation comes before the norm.  A rotation that carries ``frequencies`` is applied from
+    position * frequency, made in the kernel.
 
     ``qkv`` [N, (heads + 2 kv_heads) d]: tensor of type ``dtype`` or Partials.  Returns q as ``dtype``
     [N, heads * d]; k and v go into the caches at ``slots`` (None: not stored)."""
@@ -484,14 +544,7 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
             _require(w, name, torch.float32, (head_dim,))
     if (q_weight is None) != (k_weight is None):
         raise ValueError('q and k norms come together')
-    cos = sin = None
-    rot = 0
-    if rotation is not None:
-        cos, sin, rot = rotation.cos, rotation.sin, rotation.rot_dim
-        _require(cos, 'cos', torch.float32)
-        _require(sin, 'sin', torch.float32, cos.shape)
-        if cos.shape[1] * 2 != rot or rot > head_dim:
-            raise ValueError('rotation tables do not fit rot_dim')
+    cos, sin, rot = _rotation_arguments(rotation, head_dim)
     if slots is not None:
         _require(slots, 'slots', torch.int32, (n,))
         _check_caches(k_cache, v_cache, dtype, kv_heads, page_size, head_dim)
@@ -499,7 +552,7 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
     _check(library.load().qil_qk_norm_rope_store(
         pointer, code, splits, _ptr(q), _ptr(q_weight), _ptr(k_weight), _ptr(cos), _ptr(sin), _ptr(positions),
         _ptr(slots), _ptr(k_cache), _ptr(v_cache), n, heads, kv_heads, head_dim, rot, page_size, float(eps),
-        int(norm_dim or 0), _code(dtype), _stream()), 'qk_norm_rope_store')
+        int(norm_dim or 0), int(bool(rotate_first)), _code(dtype), _stream()), 'qk_norm_rope_store')
     return q
 
 
@@ -547,6 +600,8 @@ def decode_attention_takes(qkv, *, heads, kv_heads, head_dim, page_size, rotatio
     """Whether ``decode_attention`` takes the step: a float32 ``Partials`` q/k/v product, bfloat16 caches, sizes of
     the fused kernel."""
     rot = rotation.rot_dim if rotation is not None else 0
+    if rotation is not None and getattr(rotation, 'frequencies', None) is not None:
+        return False                                   # (the fused kernel rotates from tables)
     return isinstance(qkv, Partials) and qkv.shape[0] <= FUSED_DECODE_MOST_ROWS and dtype == torch.bfloat16 and \
         bool(library.load().qil_attn_decode_fused_takes(heads, kv_heads, head_dim, page_size, rot))
 
@@ -599,10 +654,12 @@ def decode_attention(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps,
 TILE_KEY_PARTS = None   # tests: (keys per part, parts) forces the tile kernel's key split where it takes the sizes
 
 
-def tile_key_parts(lib, dtype, n_seqs, max_query, heads, kv_heads, head_dim, page_size, table_stride, max_context):
-    """(keys per part, parts) for the matrix-core tile kernels; parts == 1: the keys in one piece."""
+def tile_key_parts(lib, dtype, n_seqs, max_query, heads, kv_heads, head_dim, page_size, table_stride, max_context,
+                   general=False):
+    """(keys per part, parts) for the matrix-core tile kernels; parts == 1: the keys in one piece.  ``general``: the
+    step runs on the general tile kernel whatever its sizes."""
     part = ctypes.c_int(0)
-    if dtype != torch.bfloat16 or not (head_dim in (64, 128) and
+    if general or dtype != torch.bfloat16 or not (head_dim in (64, 128) and
                                        lib.qil_attn_tile_bf16_takes(head_dim, page_size, table_stride)):
         parts = lib.qil_attn_tile_key_parts(n_seqs, max_query, heads, kv_heads, head_dim, max_context, _code(dtype),
                                             ctypes.byref(part))
@@ -621,7 +678,7 @@ def tile_key_parts(lib, dtype, n_seqs, max_query, heads, kv_heads, head_dim, pag
 
 def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
                     cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window,
-                    unmerged=False, tile_seqs=None):
+                    unmerged=False, tile_seqs=None, softcap=None):
     """Attention of every row of the step over its request's cached keys.
 
     ``q`` [N, heads * head_dim] (head h at columns [h d, (h + 1) d)).  Row n belongs to sequence ``row_seq[n]`` (a row of ``block_tables``) and sees keys j with
@@ -633,7 +690,12 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
     come back as ``Unmerged`` (every row alone, context in several parts) for ``linear`` to merge.
     ``tile_seqs``: the caller has put the sequences of two or more rows first and there are this many; the tile
     kernel then gets blocks for these only (None: for every sequence; those of one row leave at once).
+    ``softcap`` c: scores are scaled, then capped softly, c * tanh(score / c), before the softmax.  The kernels
+    specialised for bfloat16 heads of 64 and 128 have no cap; capped steps run on the general tile kernel.
     """
+    cap = float(softcap or 0.0)
+    if cap < 0:
+        raise ValueError('softcap must be positive')
     n = q.shape[0]
     qkv = q
     check_attention_geometry(heads=heads, kv_heads=kv_heads, head_dim=head_dim, dtype=qkv.dtype)
@@ -661,7 +723,7 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
                 raise ValueError('tile_seqs must count the sequences of two or more rows')
             n_seqs = tile_seqs
         part, parts = tile_key_parts(lib, qkv.dtype, several, max_query, heads, kv_heads,
-                                     head_dim, page_size, block_tables.shape[1], max_context)
+                                     head_dim, page_size, block_tables.shape[1], max_context, general=cap > 0)
         if parts > 1:
             # few row tiles deep in a long context: the keys in parts, one block each, merged afterwards (over all
             # rows of the step: what the merge leaves in rows that are alone is overwritten below)
@@ -669,7 +731,7 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
             merged = n if tile_seqs is None else n - single_rows.shape[0]
             workspace = torch.empty(lib.qil_attn_rows_workspace(merged, heads, head_dim, parts) // 4, dtype=torch.float32,
                                     device=qkv.device)
-            if qkv.dtype == torch.bfloat16 and head_dim in (64, 128) and \
+            if cap == 0 and qkv.dtype == torch.bfloat16 and head_dim in (64, 128) and \
                     lib.qil_attn_tile_bf16_takes(head_dim, page_size, block_tables.shape[1]):
                 _check(lib.qil_attn_tile_bf16_parts(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                                                     _ptr(block_tables), block_tables.shape[1], _ptr(cu_seqlens),
@@ -680,15 +742,15 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
                 _check(lib.qil_attn_tile_in_parts(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                                                   _ptr(block_tables), block_tables.shape[1], _ptr(cu_seqlens),
                                                   _ptr(seq_starts), _ptr(workspace), merged, n_seqs, max_query, heads,
-                                                  kv_heads, head_dim, page_size, int(window or 0), float(scale), part,
-                                                  parts, _code(qkv.dtype), _stream()), 'attn_tile_in_parts')
+                                                  kv_heads, head_dim, page_size, int(window or 0), float(scale), cap,
+                                                  part, parts, _code(qkv.dtype), _stream()), 'attn_tile_in_parts')
             _check(lib.qil_attn_merge(_ptr(workspace), _ptr(positions), None, _ptr(out), merged, heads, head_dim,
                                       int(window or 0), part, parts, _code(qkv.dtype), _stream()), 'attn_merge')
         else:
             _check(lib.qil_attn_tile(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                      block_tables.shape[1], _ptr(cu_seqlens), _ptr(seq_starts), _ptr(out), n_seqs,
                                      max_query, heads, kv_heads, head_dim, page_size, int(window or 0), float(scale),
-                                     _code(qkv.dtype), _stream()), 'attn_tile')
+                                     cap, _code(qkv.dtype), _stream()), 'attn_tile')
         rows = single_rows.shape[0]
     else:
         single_rows, rows = None, n
@@ -703,8 +765,8 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
                                        block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(single_rows),
                                        _ptr(workspace), _ptr(out), rows, heads, kv_heads, head_dim, page_size,
                                        window_arg, float(scale), part, parts, DECODE_WAVES,
-                                       int(rows * kv_heads * parts <= DECODE_PAIRS_BLOCKS and head_dim <= 128), _stream()),
-                   'attn_decode')
+                                       int(rows * kv_heads * parts <= DECODE_PAIRS_BLOCKS and head_dim <= 128), cap,
+                                       _stream()), 'attn_decode')
             if unmerged and parts > 1 and single_rows is None:
                 return Unmerged(workspace, positions, out, heads=heads, head_dim=head_dim, window=window_arg,
                                 part=part, parts=parts)
@@ -719,14 +781,14 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
                 _check(lib.qil_attn_rows_unmerged(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache),
                                                   _ptr(block_tables), block_tables.shape[1], _ptr(row_seq),
                                                   _ptr(positions), _ptr(workspace), rows, heads, kv_heads, head_dim,
-                                                  page_size, window_arg, float(scale), part, parts, _code(qkv.dtype),
+                                                  page_size, window_arg, float(scale), cap, part, parts, _code(qkv.dtype),
                                                   _stream()), 'attn_rows_unmerged')
                 return Unmerged(workspace, positions, out, heads=heads, head_dim=head_dim, window=window_arg,
                                 part=part, parts=parts)
             _check(lib.qil_attn_rows(_ptr(qkv), qkv.shape[1], _ptr(k_cache), _ptr(v_cache), _ptr(block_tables),
                                      block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(single_rows),
                                      _ptr(workspace), _ptr(out), rows, heads, kv_heads, head_dim, page_size,
-                                     window_arg, float(scale), part, parts, _code(qkv.dtype), _stream()), 'attn_rows')
+                                     window_arg, float(scale), cap, part, parts, _code(qkv.dtype), _stream()), 'attn_rows')
     return out
 
 
@@ -935,7 +997,7 @@ def latent_attention(q, *, latent, rope, page_size, block_tables, row_seq, posit
 
 # ---------------------------------------------------------------------------------------------------------------
 # Recurrences with a matrix state
-SCAN_MODES = {'decay': 0, 'mlstm': 1}
+SCAN_MODES = {'decay': 0, 'mlstm': 1, 'channel': 2}
 SCAN_BLOCKS_FROM = 32           # rows of one sequence from which a step's recurrence runs in blocks side by side
 
 
@@ -956,7 +1018,9 @@ def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, st
     ``proj`` [N, P]: a row holds the heads' queries from column ``q_offset``, keys from ``k_offset`` (heads * dim each)
     and values from ``v_offset`` (heads * vdim).  Mode 'decay': a_t = decay[h], b_t = 1.  Mode 'mlstm': exponential
     gates from ``gates`` float32 [N, 2 heads] (+ ``gate_bias`` [2 heads]; input gates first) soft-capped at ``cap``,
-    with a running maximum and a normaliser.  Queries and keys are rotated by position on their leading ``rot``
+    with a running maximum and a normaliser.  Mode 'channel': every row i of a head's S keeps a_t[i] =
+    sigmoid(z)^(1 / tau) of itself, with z = ``gates`` float32 [N, heads * dim] and tau = ``cap``; b_t = 1.
+    Queries and keys are rotated by position on their leading ``rot``
     elements (``frequencies`` [rot / 2]) and then scaled.  ``max_query``: the most rows of one sequence, if the caller
     knows it; from ``SCAN_BLOCKS_FROM`` rows on the step is worked in blocks of 64 tokens side by side (the sums of the
     blocks, their carry from block to block, the outputs), below that token by token.
@@ -983,6 +1047,10 @@ def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, st
     if mode == 'mlstm':
         _require(gates, 'gates', torch.float32, (n, 2 * heads))
         _require(gate_bias, 'gate_bias', torch.float32, (2 * heads,))
+    elif mode == 'channel':
+        _require(gates, 'gates', torch.float32, (n, heads * dim))
+        if not cap > 0:
+            raise ValueError("state_scan: mode 'channel' needs a positive tau in the place of the cap")
     else:
         _require(decay, 'decay', torch.float32, (heads,))
     if rot:
@@ -1023,4 +1091,56 @@ def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gat
     _check(library.load().qil_head_norm_gate(_ptr(o), _ptr(denominators), _ptr(gate_source), gate_source.shape[1], gate_offset, _ptr(weight),
                                              _ptr(out), n, heads, vdim, float(eps), {'sigmoid': 0, 'silu': 1}[gate],
                                              _code(out_dtype), _stream()), 'head_norm_gate')
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Routed feed-forward
+def moe_route(x, router, correction, *, groups, keep, top, renormalize=False):
+    """x [N, width] (model type), router float32 [outputs, width], correction float32 [outputs] or None ->
+    (chosen int32 [N, top], weights float32 [N, top]): softmax scores over all outputs in float32; the choice goes
+    by score + correction among the outputs of the ``keep`` best of ``groups`` equal groups of neighbours (a group's
+    score: its best choice score); the weights are the chosen outputs' scores (divided by their sum if asked)."""
+    n, width = x.shape
+    _require(x, 'x')
+    outputs = router.shape[0]
+    _require(router, 'router', torch.float32, (outputs, width))
+    if correction is not None:
+        _require(correction, 'correction', torch.float32, (outputs,))
+    lib = library.load()
+    if not lib.qil_moe_takes(width, outputs, 0, groups, keep, top):
+        raise UnsupportedShape(f'moe_route: {outputs} outputs in {groups} groups ({keep} kept), top {top}, width {width}')
+    chosen = torch.empty((n, top), dtype=torch.int32, device=x.device)
+    weights = torch.empty((n, top), dtype=torch.float32, device=x.device)
+    _check(lib.qil_moe_route(_ptr(x), _code(x.dtype), _ptr(router), _ptr(correction), _ptr(chosen), _ptr(weights), n, width,
+                             outputs, groups, keep, top, int(bool(renormalize)), _stream()), 'moe_route')
+    return chosen, weights
+
+
+def moe_experts(x, chosen, weights, gate_up, down, *, activation, limit=0.0, alpha=1.0):
+    """The weighted sum of the chosen experts' outputs, float32 [N, width].  ``gate_up`` [experts, 2, ff, width] (an
+    expert's gate rows, then its up rows), ``down`` [experts, width, ff], both of x's type; an expert computes
+    down(act(gate x, up x)) with ``activation`` of ``GATE_FUNCTIONS``.  A chosen index from ``experts`` on is an
+    identity expert: its output is x itself.  The pairs (token, chosen expert) are grouped by expert on the device;
+    the host sees no routing result, so a step may be captured into a graph."""
+    n, width = x.shape
+    top = chosen.shape[1]
+    _require(x, 'x')
+    _require(chosen, 'chosen', torch.int32, (n, top))
+    _require(weights, 'weights', torch.float32, (n, top))
+    experts, ff = gate_up.shape[0], gate_up.shape[2]
+    _require(gate_up, 'gate_up', x.dtype, (experts, 2, ff, width))
+    _require(down, 'down', x.dtype, (experts, width, ff))
+    lib = library.load()
+    pairs = n * top
+    tile_rows = lib.qil_moe_tile_rows(pairs, experts)
+    max_tiles = lib.qil_moe_max_tiles(pairs, experts, tile_rows)
+    scratch = torch.empty(3 * max_tiles + pairs, dtype=torch.int32, device=x.device)
+    hidden = torch.empty((pairs, ff), dtype=x.dtype, device=x.device)
+    y = torch.empty((pairs, width), dtype=torch.float32, device=x.device)
+    out = torch.empty((n, width), dtype=torch.float32, device=x.device)
+    _check(lib.qil_moe_experts(_ptr(x), _code(x.dtype), _ptr(chosen), _ptr(weights), _ptr(gate_up), _ptr(down),
+                               _ptr(scratch), scratch[3 * max_tiles:].data_ptr(), _ptr(hidden), _ptr(y), _ptr(out), n, width,
+                               ff, experts, top, tile_rows, max_tiles, GATE_FUNCTIONS[activation], float(limit),
+                               float(alpha), _stream()), 'moe_experts')
     return out

@@ -208,22 +208,22 @@ def _declare(lib):
     lib.qil_planned_compute_units.argtypes = []
     lib.qil_planned_compute_units.restype = i
     lib.qil_device_info.restype = i
-    lib.qil_embed.argtypes = [p, p, p, i, i, i, p]
+    lib.qil_embed.argtypes = [p, p, p, i, i, f, i, p]
     lib.qil_add_rmsnorm.argtypes = [p, p, i, i, i, p, p, p, i, i, f, i, i, p]
     lib.qil_silu_mul.argtypes = [p, i, i, p, i, i, i, i, p]
     lib.qil_add_bias.argtypes = [p, p, i, i, i, p]
-    lib.qil_qk_norm_rope_store.argtypes = [p, i, i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i, i, p]
+    lib.qil_qk_norm_rope_store.argtypes = [p, i, i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, p]
     lib.qil_attn_rows_workspace.argtypes = [i, i, i, i]
     lib.qil_attn_rows_workspace.restype = z
-    lib.qil_attn_rows.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, p]
+    lib.qil_attn_rows.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, f, i, i, i, p]
     lib.qil_attn_merge.argtypes = [p, p, p, p, i, i, i, i, i, i, i, p]
     lib.qil_attn_decode_fused_takes.argtypes = [i, i, i, i, i]
     lib.qil_attn_decode_fused_takes.restype = i
     lib.qil_attn_decode_fused.argtypes = [p, i, p, p, f, p, p, i, i, p, p, p, i, p, p, p, p, i, i, i, i, i, i, f, i, i, i, i, p]
     lib.qil_attn_decode_takes.argtypes = [i, i, i, i]
     lib.qil_attn_decode_takes.restype = i
-    lib.qil_attn_decode.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, i, p]
-    lib.qil_attn_tile.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, f, i, p]
+    lib.qil_attn_decode.argtypes = [p, i, p, p, p, i, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i, i, f, p]
+    lib.qil_attn_tile.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, f, f, i, p]
     lib.qil_gemm_f32.argtypes = [p, p, p, p, i, i, i, i, p]
     lib.qil_gemm_f32_splits.argtypes = [i, i, i]
     lib.qil_gemm_f32_waves.argtypes = [i, i, i, i]
@@ -236,7 +236,7 @@ def _declare(lib):
     lib.qil_gemm_f32_gated_takes.restype = i
     lib.qil_gemm_f32_gated.argtypes = [p, i, i, p, p, i, i, i, i, p]
     lib.qil_gemm_f32_gated.restype = i
-    lib.qil_attn_rows_unmerged.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, f, i, i, i, p]
+    lib.qil_attn_rows_unmerged.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, f, f, i, i, i, p]
     lib.qil_attn_rows_unmerged.restype = i
     lib.qil_gemm_f32_mfma.argtypes = [p, p, p, p, i, i, i, i, p]
     lib.qil_gemm_f32_mfma_takes.argtypes = [i, i, i, i]
@@ -255,7 +255,7 @@ def _declare(lib):
     lib.qil_attn_tile_bf16_parts.restype = i
     lib.qil_attn_tile_key_parts.argtypes = [i, i, i, i, i, i, i, ctypes.POINTER(ctypes.c_int)]
     lib.qil_attn_tile_key_parts.restype = i
-    lib.qil_attn_tile_in_parts.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, i, f, i, i, i, p]
+    lib.qil_attn_tile_in_parts.argtypes = [p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, i, f, f, i, i, i, p]
     lib.qil_attn_tile_in_parts.restype = i
     lib.qil_attn_tile_waves.argtypes = [i]
     lib.qil_attn_tile_waves.restype = None
@@ -317,6 +317,18 @@ def _declare(lib):
     for name in ('qil_add_norm', 'qil_gated_act', 'qil_latent_prepare', 'qil_head_product', 'qil_rotate_tail',
                  'qil_latent_attention', 'qil_state_scan', 'qil_head_norm_gate'):
         getattr(lib, name).restype = i
+    lib.qil_post_norm_add_norm.argtypes = [p, p, i, i, i, p, f, p, p, p, i, i, f, i, i, p]
+    lib.qil_post_norm_add_norm.restype = i
+    lib.qil_moe_takes.argtypes = [i, i, i, i, i, i]
+    lib.qil_moe_takes.restype = i
+    lib.qil_moe_route.argtypes = [p, i, p, p, p, p, i, i, i, i, i, i, i, p]
+    lib.qil_moe_route.restype = i
+    lib.qil_moe_tile_rows.argtypes = [i, i]
+    lib.qil_moe_tile_rows.restype = i
+    lib.qil_moe_max_tiles.argtypes = [i, i, i]
+    lib.qil_moe_max_tiles.restype = i
+    lib.qil_moe_experts.argtypes = [p, i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, f, f, p]
+    lib.qil_moe_experts.restype = i
     lib.qil_sample.argtypes = [p, p, p, p, p, p, p, i, i, p]
     lib.qil_sample_workspace.argtypes = [i, i]
     lib.qil_sample_workspace.restype = z

@@ -7,11 +7,12 @@ from .attention import Attention
 from .latent_attention import LatentAttention
 from .recurrent import MatrixMemory
 from .mlp import GatedMLP
-from .block import PreNormBlock
+from .moe import RoutedExperts
+from .block import PreNormBlock, SandwichBlock
 from .embedding import Embedding, LMHead
 from .model import CausalLM, ScheduleEntry
 
 __all__ = ['ParamSpec', 'KVNeed', 'PagedNeed', 'StateNeed', 'Part', 'Norm', 'PositionEncoding', 'Rotation', 'Mixer',
            'FeedForward', 'Block', 'RMSNorm', 'LayerNorm', 'Rotary', 'RotaryFrequencies', 'Attention',
-           'LatentAttention', 'MatrixMemory', 'GatedMLP', 'PreNormBlock',
+           'LatentAttention', 'MatrixMemory', 'GatedMLP', 'RoutedExperts', 'PreNormBlock', 'SandwichBlock',
            'Embedding', 'LMHead', 'CausalLM', 'ScheduleEntry']

@@ -22,31 +22,48 @@ class Attention(Mixer):
     of queries, keys and values are then exact zeros, which add nothing to a score or to the output; the head norm's
     mean runs over the true size (``norm_dim``), the rotation over the true size's pairs, and the scale is the
     caller's.  The cache holds the padded size.
+
+    What a design may change beyond sizes: ``value_dim`` (values of another size than queries and keys: every head is
+    padded with zeros to the larger of the two, so keys and values share the kernels' one head size; the output
+    matrix gets zero columns for the padding); ``softcap`` c (scores become c * tanh(score / c) after the scale);
+    ``qk_norm_weights=False`` (the head norms divide by the root mean square and multiply by nothing: the part
+    declares no norm tensors); ``norm_after_rotation`` (queries and keys are rotated first and normed then).
+    ``position`` may be a ``Rotary`` (tables) or a ``RotaryFrequencies`` (the kernels make the angles from the
+    positions, which no table bounds).
     """
     graph_safe = True
     takes_lazy_norm = True       # h goes into ops.linear only, which takes a norm not computed yet
 
     def __init__(self, *, width, heads, kv_heads, head_dim, bias, qk_norm_eps, scale,
-                 position=None, window=None, dtype=torch.bfloat16):
+                 position=None, window=None, dtype=torch.bfloat16, value_dim=None, softcap=None, qk_norm_weights=True,
+                 norm_after_rotation=False):
         super().__init__()
         if heads % kv_heads:
             raise ValueError('heads must be a multiple of kv_heads')
         self.width, self.heads, self.kv_heads, self.head_dim = width, heads, kv_heads, head_dim
         self.bias, self.qk_norm_eps, self.scale = bool(bias), qk_norm_eps, float(scale)
         self.position, self.window, self.dtype = position, window, dtype
+        self.value_dim = head_dim if value_dim is None else value_dim
+        self.softcap = None if softcap is None else float(softcap)
+        self.qk_norm_weights, self.norm_after_rotation = bool(qk_norm_weights), bool(norm_after_rotation)
+        if self.softcap is not None and not self.softcap > 0:
+            raise ValueError('softcap must be positive')
+        if type(self.value_dim) is not int or self.value_dim < 1:
+            raise ops.UnsupportedShape(f'value_dim {self.value_dim!r} must be a positive integer')
         if head_dim < 2 or head_dim % 2:
             raise ops.UnsupportedShape(f'head_dim {head_dim} must be even')
-        self.padded_dim = -(-head_dim // 8) * 8               # what the kernels and the cache see
+        self.padded_dim = -(-max(head_dim, self.value_dim) // 8) * 8    # what the kernels and the cache see
         ops.check_attention_geometry(heads=heads, kv_heads=kv_heads, head_dim=self.padded_dim, dtype=dtype)
 
     def param_specs(self):
         q, kv, d = self.heads * self.head_dim, self.kv_heads * self.head_dim, self.head_dim
+        v, o = self.kv_heads * self.value_dim, self.heads * self.value_dim
         specs = {'q_proj.weight': ParamSpec((q, self.width)), 'k_proj.weight': ParamSpec((kv, self.width)),
-                 'v_proj.weight': ParamSpec((kv, self.width)), 'o_proj.weight': ParamSpec((self.width, q))}
+                 'v_proj.weight': ParamSpec((v, self.width)), 'o_proj.weight': ParamSpec((self.width, o))}
         if self.bias:   # o_proj gets a bias too (qil/model.py:35)
             specs.update({'q_proj.bias': ParamSpec((q,), 'vector'), 'k_proj.bias': ParamSpec((kv,), 'vector'),
-                          'v_proj.bias': ParamSpec((kv,), 'vector'), 'o_proj.bias': ParamSpec((self.width,), 'vector')})
-        if self.qk_norm_eps is not None:
+                          'v_proj.bias': ParamSpec((v,), 'vector'), 'o_proj.bias': ParamSpec((self.width,), 'vector')})
+        if self.qk_norm_eps is not None and self.qk_norm_weights:
             specs.update({'q_norm.weight': ParamSpec((d,), 'vector', 'one_plus_normal'),
                           'k_norm.weight': ParamSpec((d,), 'vector', 'one_plus_normal')})
         return specs
@@ -54,9 +71,10 @@ class Attention(Mixer):
     def cache_need(self):
         return KVNeed(self.kv_heads, self.padded_dim, self.window)
 
-    def _pad_heads(self, tensor, axis=0):
-        """``tensor`` with every head's ``head_dim`` entries along ``axis`` followed by zeros up to ``padded_dim``."""
-        d, dp = self.head_dim, self.padded_dim
+    def _pad_heads(self, tensor, axis=0, d=None):
+        """``tensor`` with every head's ``d`` (default ``head_dim``) entries along ``axis`` followed by zeros up to
+        ``padded_dim``."""
+        d, dp = d or self.head_dim, self.padded_dim
         if d == dp:
             return tensor
         count = tensor.shape[axis] // d
@@ -71,28 +89,40 @@ class Attention(Mixer):
 
     def finalize(self):
         p = self.p
-        self.w_qkv = torch.cat([self._pad_heads(p.pop(name)) for name in
-                                ('q_proj.weight', 'k_proj.weight', 'v_proj.weight')]).contiguous()
-        self.b_qkv = (torch.cat([self._pad_heads(p.pop(name)) for name in
-                                 ('q_proj.bias', 'k_proj.bias', 'v_proj.bias')]).contiguous() if self.bias else None)
+        sizes = (self.head_dim, self.head_dim, self.value_dim)
+        self.w_qkv = torch.cat([self._pad_heads(p.pop(name), d=d) for name, d in
+                                zip(('q_proj.weight', 'k_proj.weight', 'v_proj.weight'), sizes)]).contiguous()
+        self.b_qkv = (torch.cat([self._pad_heads(p.pop(name), d=d) for name, d in
+                                 zip(('q_proj.bias', 'k_proj.bias', 'v_proj.bias'), sizes)]).contiguous()
+                      if self.bias else None)
         p['qkv_proj.weight'] = self.w_qkv
         if self.bias:
             p['qkv_proj.bias'] = self.b_qkv
+        if self.padded_dim != self.value_dim:
+            p['o_proj.weight'] = self._pad_heads(p['o_proj.weight'], axis=1, d=self.value_dim).contiguous()
         if self.padded_dim != self.head_dim:
-            p['o_proj.weight'] = self._pad_heads(p['o_proj.weight'], axis=1).contiguous()
             for name in ('q_norm.weight', 'k_norm.weight'):
                 if name in p:
                     p[name] = self._pad_heads(p[name]).contiguous()
+        if self.qk_norm_eps is not None and not self.qk_norm_weights:       # a norm that multiplies by nothing
+            self._ones = torch.ones(self.padded_dim, dtype=torch.float32, device=self.w_qkv.device)
+        if self.position is not None:
+            self.position.rotation()                     # device tensors are made here, not in a step that may be captured
 
     def forward(self, h, ctx, cache):
         p = self.p
         qkv = ops.linear(h, self.w_qkv, self.b_qkv, partials=True)
         rotation = self.position.rotation() if self.position is not None else None
-        norms = dict(q_weight=p.get('q_norm.weight'), k_weight=p.get('k_norm.weight'),
-                     eps=self.qk_norm_eps if self.qk_norm_eps is not None else 0.0)
+        if self.qk_norm_eps is not None and not self.qk_norm_weights:
+            norms = dict(q_weight=self._ones, k_weight=self._ones, eps=self.qk_norm_eps)
+        else:
+            norms = dict(q_weight=p.get('q_norm.weight'), k_weight=p.get('k_norm.weight'),
+                         eps=self.qk_norm_eps if self.qk_norm_eps is not None else 0.0)
         sizes = dict(heads=self.heads, kv_heads=self.kv_heads, head_dim=self.padded_dim)
-        # (the kernel that makes its queries itself norms over the whole head it sees: not for padded heads)
-        if ctx.max_query == 1 and self.padded_dim == self.head_dim and \
+        # (the kernel that makes its queries itself norms over the whole head it sees, norms before it rotates and
+        # caps nothing: not for padded heads, and not for designs that differ there)
+        if ctx.max_query == 1 and self.padded_dim == self.head_dim and self.softcap is None and \
+                not self.norm_after_rotation and \
                 ops.decode_attention_takes(qkv, page_size=cache.page_size, rotation=rotation, dtype=self.dtype, **sizes):
             # every row alone in its sequence: norm, rotation and cache write happen inside the attention kernel
             attended = ops.decode_attention(
@@ -103,11 +133,11 @@ class Attention(Mixer):
         q = ops.qk_norm_rope_store(
             qkv, rotation=rotation, positions=ctx.positions, slots=cache.slots if cache.writes else None,
             k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size, dtype=self.dtype, norm_dim=self.head_dim,
-            **sizes, **norms)
+            rotate_first=self.norm_after_rotation, **sizes, **norms)
         attended = ops.paged_attention(
             q, k_cache=cache.k, v_cache=cache.v, page_size=cache.page_size,
             block_tables=cache.block_tables, row_seq=ctx.row_seq, positions=ctx.positions,
             cu_seqlens=ctx.cu_seqlens, seq_starts=ctx.seq_starts, single_rows=ctx.single_rows, n_seqs=ctx.n_seqs,
             max_query=ctx.max_query, max_context=ctx.max_context, tile_seqs=ctx.tile_seqs,
-            scale=self.scale, window=self.window, unmerged=True, **sizes)
+            scale=self.scale, window=self.window, unmerged=True, softcap=self.softcap, **sizes)
         return ops.linear(attended, p['o_proj.weight'], p.get('o_proj.bias'), partials=True)

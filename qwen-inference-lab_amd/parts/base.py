@@ -7,8 +7,8 @@ out once in ``finalize()``, and computes with the kernels of ``qil_amd.ops``.
 
 Tensor kinds (``ParamSpec.kind``):
   matrix  -> stored in the model's dtype (bfloat16 or float32)
-  vector  -> norm scales and biases; always float32 on the device, which holds a
-             bfloat16 or a float32 checkpoint value exactly
+  vector  -> norm scales and biases, and small matrices whose products are float32 in every model (a router);
+             always float32 on the device, which holds a bfloat16 or a float32 checkpoint value exactly
   table   -> integer tables; int32
 """
 from dataclasses import dataclass
@@ -19,6 +19,14 @@ class ParamSpec:
     shape: tuple
     kind: str = 'matrix'          # matrix | vector | table
     init: str = 'normal'          # normal | one_plus_normal | zeros
+    free: tuple = ()              # axes whose size the checkpoint decides (no configuration key gives it); the size
+                                  # in ``shape`` is what random weights get, and the part checks in ``finalize`` that
+                                  # the sizes it was given fit each other
+
+    def fits(self, shape):
+        shape = tuple(shape)
+        return len(shape) == len(self.shape) and all(a == b or axis in self.free
+                                                     for axis, (a, b) in enumerate(zip(shape, self.shape)))
 
 
 @dataclass(frozen=True)
@@ -61,7 +69,7 @@ class Part:
 
     def set_param(self, name, tensor):
         spec = self.param_specs()[name]
-        if tuple(tensor.shape) != tuple(spec.shape):
+        if not spec.fits(tensor.shape):
             raise ValueError(f'{type(self).__name__}.{name}: shape {tuple(tensor.shape)} != {tuple(spec.shape)}')
         self.p[name] = tensor
 
@@ -107,9 +115,10 @@ class PositionEncoding(Part):
 
 @dataclass(frozen=True)
 class Rotation:
-    cos: object            # float32 [positions, rot_dim/2]
+    cos: object            # float32 [positions, rot_dim/2]; None with ``frequencies``
     sin: object
     rot_dim: int           # leading rot_dim elements of each head are rotated, pairs (i, i + rot_dim/2)
+    frequencies: object = None   # float32 [rot_dim/2]: the kernels make the angle position * frequency themselves
 
 
 class Mixer(Part):

@@ -51,3 +51,40 @@ class PreNormBlock(Block):
         if self.ffn is None:
             return mixed
         return self.ffn.forward(self.ffn_norm.forward(stream, mixed, self.dtype, delta_scale=m))
+
+
+class SandwichBlock(Block):
+    """A norm before and a norm after every sub-layer: x <- x + post(sublayer(pre(x))), mixer then feed-forward (or
+    the mixer alone).  The stream and both norms' statistics are float32; a sub-layer's output leaves the block as an
+    ``ops.PostNormed`` (not yet normed, not yet added), and the norm that follows, this block's or the next one's or
+    the model's last, makes the post norm, the sum and its own norm in one kernel."""
+
+    def __init__(self, *, mixer_norm, mixer, mixer_post_norm, ffn_norm=None, ffn=None, ffn_post_norm=None, dtype, names=None):
+        super().__init__()
+        self.mixer_norm, self.mixer, self.mixer_post_norm = mixer_norm, mixer, mixer_post_norm
+        self.ffn_norm, self.ffn, self.ffn_post_norm, self.dtype = ffn_norm, ffn, ffn_post_norm, dtype
+        if len({ffn is None, ffn_norm is None, ffn_post_norm is None}) != 1:
+            raise ValueError('a feed-forward and its two norms come together')
+        self._names = names or dict(mixer_norm='mixer_norm', mixer='mixer', mixer_post_norm='mixer_post_norm',
+                                    ffn_norm='ffn_norm', ffn='ffn', ffn_post_norm='ffn_post_norm')
+
+    def parts(self):
+        n = self._names
+        out = {n['mixer_norm']: self.mixer_norm, n['mixer']: self.mixer, n['mixer_post_norm']: self.mixer_post_norm}
+        if self.ffn is not None:
+            out.update({n['ffn_norm']: self.ffn_norm, n['ffn']: self.ffn, n['ffn_post_norm']: self.ffn_post_norm})
+        return out
+
+    @staticmethod
+    def _post(norm, value):
+        return ops.PostNormed(value, norm.p['weight'], norm.eps)
+
+    def forward(self, stream, pending, ctx, cache):
+        if isinstance(pending, ops.Added):                     # the stream is complete
+            pending = None
+        h = self.mixer_norm.forward(stream, pending, self.dtype)
+        mixed = self._post(self.mixer_post_norm, self.mixer.forward(h, ctx, cache))
+        if self.ffn is None:
+            return mixed
+        h = self.ffn_norm.forward(stream, mixed, self.dtype)
+        return self._post(self.ffn_post_norm, self.ffn.forward(h))

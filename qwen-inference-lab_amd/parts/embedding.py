@@ -4,17 +4,17 @@ from .. import ops
 
 
 class Embedding(Part):
-    """stream[n] = float32(table[token[n]]), no scaling (qil/model.py:126)."""
+    """stream[n] = float32(table[token[n]]) * scale; no scaling (scale 1) in qil/model.py:126."""
 
-    def __init__(self, vocab, width):
+    def __init__(self, vocab, width, scale=1.0):
         super().__init__()
-        self.vocab, self.width = vocab, width
+        self.vocab, self.width, self.scale = vocab, width, float(scale)
 
     def param_specs(self):
         return {'weight': ParamSpec((self.vocab, self.width))}
 
     def forward(self, token_ids):
-        return ops.embed(token_ids, self.p['weight'])
+        return ops.embed(token_ids, self.p['weight'], self.scale)
 
     def forward_step(self, ctx):
         """The float32 stream [N, width] of a step's rows.  What the model calls; an embedding that also needs

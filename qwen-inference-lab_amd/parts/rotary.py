@@ -49,6 +49,9 @@ class RotaryFrequencies(PositionEncoding):
             raise ValueError('the base must be positive')
         self._frequencies = None
 
+    def rotation(self):
+        return Rotation(None, None, self.rot_dim, self.frequencies())
+
     def frequencies(self):
         if self._frequencies is None:
             values = [self.base ** (-2.0 * i / self.rot_dim) for i in range(self.rot_dim // 2)]

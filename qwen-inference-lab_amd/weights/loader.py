@@ -52,7 +52,7 @@ def load_weights(model, directory):
                 spec = part.param_specs()[local]
                 view = shard.get_slice(name)
                 shape, stored = tuple(view.get_shape()), view.get_dtype()
-                if shape != tuple(spec.shape):
+                if not spec.fits(shape):
                     wrong_shape.append(f'{name}: file {list(shape)}, model {list(spec.shape)}')
                 if stored not in (_INTS if spec.kind == 'table' else _FLOATS):
                     wrong_type.append(f'{name}: stored as {stored}')
