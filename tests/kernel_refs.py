@@ -17,8 +17,8 @@ def _round(x, dtype):
     return x.to(dtype).to(torch.float32)
 
 
-def embed(token_ids, table):
-    return table[token_ids.long()].to(torch.float32)
+def embed(token_ids, table, scale=1.0):
+    return table[token_ids.long()].to(torch.float32) * scale
 
 
 def _norm(x, weight, eps, out_dtype):
@@ -26,16 +26,24 @@ def _norm(x, weight, eps, out_dtype):
     return (_round(n, out_dtype) * weight).to(out_dtype)
 
 
+def _delta(delta):
+    """What a pending sub-layer output adds: itself, or (``PostNormed``) its RMS norm in float32, unrounded."""
+    if hasattr(delta, 'value') and hasattr(delta, 'eps'):
+        x = _value(delta.value).to(torch.float32)
+        return x * torch.rsqrt(x.square().mean(dim=-1, keepdim=True) + delta.eps) * delta.weight
+    return _value(delta).to(torch.float32)
+
+
 def add_rmsnorm(stream, delta, weight, eps, out_dtype):
     if delta is not None:
-        stream += _value(delta).to(torch.float32)
+        stream += _delta(delta)
     return _norm(stream, weight, eps, out_dtype)
 
 
 def rows_rmsnorm(stream, delta, rows, weight, eps, out_dtype):
     x = stream[rows.long()]
     if delta is not None:
-        x = x + _value(delta)[rows.long()].to(torch.float32)
+        x = x + _delta(delta)[rows.long()]
     return _norm(x, weight, eps, out_dtype)
 
 
@@ -75,22 +83,32 @@ def silu_mul(gate_up, out_dtype=None, interleaved=False):
 
 
 def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, slots,
-                       k_cache, v_cache, page_size, dtype, norm_dim=None):
+                       k_cache, v_cache, page_size, dtype, norm_dim=None, rotate_first=False):
     qkv = _value(qkv)
     n, d = qkv.shape[0], head_dim
     x = qkv.view(n, heads + 2 * kv_heads, d)
     q, k, v = x[:, :heads].to(torch.float32), x[:, heads:heads + kv_heads].to(torch.float32), x[:, heads + kv_heads:]
 
-    def shape(t, weight):
-        if weight is not None:
-            t = _round(t * torch.rsqrt(t.square().sum(dim=-1, keepdim=True) / (norm_dim or d) + eps), dtype) * weight
-        if rotation is not None:
-            rot, half = rotation.rot_dim, rotation.rot_dim // 2
+    def normed(t, weight):
+        if weight is None:
+            return t
+        return _round(t * torch.rsqrt(t.square().sum(dim=-1, keepdim=True) / (norm_dim or d) + eps), dtype) * weight
+
+    def turned(t):
+        if rotation is None:
+            return t
+        rot, half = rotation.rot_dim, rotation.rot_dim // 2
+        if getattr(rotation, 'frequencies', None) is not None:
+            angle = positions.to(torch.float32)[:, None] * rotation.frequencies[None, :]
+            c, s = angle.cos()[:, None, :], angle.sin()[:, None, :]
+        else:
             c = rotation.cos[positions.long()][:, None, :]
             s = rotation.sin[positions.long()][:, None, :]
-            left, right = t[..., :half], t[..., half:rot]
-            t = torch.cat((left * c - right * s, left * s + right * c, t[..., rot:]), dim=-1)
-        return t.to(dtype)
+        left, right = t[..., :half], t[..., half:rot]
+        return torch.cat((left * c - right * s, left * s + right * c, t[..., rot:]), dim=-1)
+
+    def shape(t, weight):
+        return (normed(turned(t), weight) if rotate_first else turned(normed(t, weight))).to(dtype)
 
     if slots is not None:
         page, offset = slots.long() // page_size, slots.long() % page_size
@@ -101,7 +119,7 @@ def qk_norm_rope_store(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, ep
 
 def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size, block_tables, row_seq, positions,
                     cu_seqlens, seq_starts, single_rows, n_seqs, max_query, max_context, scale, window,
-                    unmerged=False, tile_seqs=None, accumulate=torch.float32):
+                    unmerged=False, tile_seqs=None, softcap=None, accumulate=torch.float32):
     n, d, g = q.shape[0], head_dim, heads // kv_heads
     qkv = q
     q = q.reshape(n, heads, d).to(accumulate)
@@ -116,6 +134,8 @@ def paged_attention(q, *, heads, kv_heads, head_dim, k_cache, v_cache, page_size
         keys = keys.repeat_interleave(g, dim=1)
         values = values.repeat_interleave(g, dim=1)
         scores = torch.einsum('hd,jhd->hj', q[row], keys) * scale
+        if softcap:
+            scores = softcap * torch.tanh(scores / softcap)
         out[row] = torch.einsum('hj,jhd->hd', torch.softmax(scores, dim=-1), values)
     return out.reshape(n, heads * d).to(qkv.dtype)
 
@@ -274,6 +294,12 @@ def state_scan(proj, *, mode, heads, dim, vdim, q_offset, k_offset, v_offset, st
                 log_keep = torch.nn.functional.logsigmoid(cap * torch.tanh(pre[heads:] / cap))
                 now = torch.maximum(log_keep + top, log_in)
                 a, b, top = torch.exp(log_keep + top - now), torch.exp(log_in - now), now
+            elif mode == 'channel':                  # a decay per row of the memory: sigmoid(z)^(1 / tau)
+                a = torch.exp(torch.nn.functional.logsigmoid(gates[lo + t].view(heads, dim)) / cap)[:, :, None]
+                b = torch.ones(heads)
+                memory = a * memory + ks[t][:, :, None] * v[lo + t][:, None, :]
+                out[lo + t] = torch.einsum('hdv,hd->hv', memory, qs[t])
+                continue
             else:
                 a, b = decay, torch.ones(heads)
             memory = a[:, None, None] * memory + b[:, None, None] * ks[t][:, :, None] * v[lo + t][:, None, :]
@@ -301,7 +327,40 @@ def head_norm_gate(o, gate_source, *, gate_offset, heads, vdim, weight, eps, gat
     return (unit * (torch.sigmoid(g) if gate == 'sigmoid' else g * torch.sigmoid(g))).to(out_dtype)
 
 
-ALL = dict(embed=embed, add_rmsnorm=add_rmsnorm, rows_rmsnorm=rows_rmsnorm, linear=linear, gated_linear=gated_linear, silu_mul=silu_mul,
+def moe_route(x, router, correction, *, groups, keep, top, renormalize=False):
+    scores = torch.softmax(x.to(torch.float32) @ router.t(), dim=-1)
+    choice = scores + correction if correction is not None else scores.clone()
+    n, outputs = scores.shape
+    if groups > 1 and keep < groups:
+        best = choice.view(n, groups, outputs // groups).max(dim=-1).values
+        kept = torch.zeros_like(best, dtype=torch.bool).scatter_(1, best.topk(keep, dim=-1).indices, True)
+        choice = choice.masked_fill(~kept.repeat_interleave(outputs // groups, dim=1), float('-inf'))
+    chosen = choice.topk(top, dim=-1).indices
+    weights = scores.gather(1, chosen)
+    if renormalize:
+        weights = weights / weights.sum(dim=-1, keepdim=True)
+    return chosen.to(torch.int32), weights
+
+
+def moe_experts(x, chosen, weights, gate_up, down, *, activation, limit=0.0, alpha=1.0):
+    """float32 [N, width]; the hidden activations pass through x's type as the kernel's do."""
+    n, width = x.shape
+    experts = gate_up.shape[0]
+    xf = x.to(torch.float32)
+    out = torch.zeros((n, width), dtype=torch.float32)
+    for row in range(n):
+        for slot in range(chosen.shape[1]):
+            e = int(chosen[row, slot])
+            if e >= experts:
+                out[row] += weights[row, slot] * xf[row]
+                continue
+            g, u = gate_up[e, 0].to(torch.float32) @ xf[row], gate_up[e, 1].to(torch.float32) @ xf[row]
+            hidden = _round(_gate(g, u, activation, limit, alpha), x.dtype)
+            out[row] += weights[row, slot] * (down[e].to(torch.float32) @ hidden)
+    return out
+
+
+ALL = dict(moe_route=moe_route, moe_experts=moe_experts, embed=embed, add_rmsnorm=add_rmsnorm, rows_rmsnorm=rows_rmsnorm, linear=linear, gated_linear=gated_linear, silu_mul=silu_mul,
            qk_norm_rope_store=qk_norm_rope_store, paged_attention=paged_attention, sample=sample,
            add_norm=add_norm, rows_norm=rows_norm, gated_act=gated_act, latent_prepare=latent_prepare, head_product=head_product,
            latent_query=latent_query, latent_attention=latent_attention, state_scan_slot=state_scan_slot, state_scan=state_scan,

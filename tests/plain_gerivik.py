@@ -128,3 +128,82 @@ def logits(tokens, weights, config, dtype=torch.float64, streams=None):
         if streams is not None:
             streams.append(x.clone())
     return rms_norm(x, w['final.norm'], eps) @ w['head'].t()
+
+
+def greedy(prompt, count, weights, config, dtype=torch.float64):
+    tokens = list(prompt)
+    for _ in range(count):
+        tokens.append(int(logits(tokens, weights, config, dtype)[-1].argmax()))
+    return tokens[len(prompt):]
+
+
+# ---------------------------------------------------------------------------------------------- configurations
+def moe_mlp(*, ff, limit, experts, identity, top, count=1, keep=1):
+    return dict(kind='moe', expert=dict(ff=ff, limit=limit),
+                router=dict(experts=experts, identity=identity, top=top, groups=dict(count=count, keep=keep)))
+
+
+def attention_layer(*, heads, kv_heads, dim, vdim, rot_dims, scale, softcap, base=10000.0, mlp=None):
+    return dict(type='attention', mlp=mlp,
+                mixer=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, rot=dict(base=base, dims=rot_dims), scale=scale,
+                           softcap=softcap))
+
+
+def gla_layer(*, heads, dim, vdim, tau, mlp=None):
+    return dict(type='gla', mlp=mlp, mixer=dict(heads=heads, dim=dim, vdim=vdim, tau=tau))
+
+
+def shared(config_layers, source):
+    """One more run of layer ``source`` with a cache of its own."""
+    return dict(config_layers[source], weights_of=source)
+
+
+def make_config(layers, *, vocab, width, scale=1.0, eps=1e-6):
+    return dict(architecture='Gerivik', vocab=vocab, width=width, embedding=dict(scale=scale), layers=layers,
+                norm=dict(eps=eps))
+
+
+def random_weights(config, seed, spread=1.0, decay_rank=5, decay_bias=2.0):
+    """Tensors under the checkpoint's names, rounded to bfloat16 values (a float32 and a bfloat16 engine then read the
+    same numbers).  ``spread`` scales the matrices around 1 / sqrt(fan-in); the decays' biases are shifted up so that
+    the memories keep what they hold for tens of tokens."""
+    g = torch.Generator().manual_seed(seed)
+    width = config['width']
+
+    def matrix(rows, columns, gain=1.0):
+        return (torch.randn(rows, columns, generator=g) * (spread * gain / math.sqrt(columns))).to(torch.bfloat16).to(torch.float64)
+
+    def scale(size):
+        return (1.0 + 0.1 * torch.randn(size, generator=g)).to(torch.bfloat16).to(torch.float64)
+
+    w = {'embed': matrix(config['vocab'], width, math.sqrt(width)), 'final.norm': scale(width), 'head': matrix(config['vocab'], width)}
+    for index, layer in enumerate(config['layers']):
+        if 'weights_of' in layer:
+            continue
+        pre, m = f'l{index}.', layer['mixer']
+        w[pre + 'norm1'], w[pre + 'norm1b'] = scale(width), scale(width)
+        if layer['type'] == 'attention':
+            w[pre + 'mix.q'] = matrix(m['heads'] * m['dim'], width, 2.0)
+            w[pre + 'mix.k'] = matrix(m['kv_heads'] * m['dim'], width, 2.0)
+            w[pre + 'mix.v'] = matrix(m['kv_heads'] * m['vdim'], width)
+            w[pre + 'mix.o'] = matrix(width, m['heads'] * m['vdim'])
+        else:
+            hd, hv = m['heads'] * m['dim'], m['heads'] * m['vdim']
+            for name, rows in (('q', hd), ('k', hd), ('v', hv), ('g', hv)):
+                w[pre + 'mix.' + name] = matrix(rows, width)
+            w[pre + 'mix.o'] = matrix(width, hv)
+            w[pre + 'mix.norm'] = scale(m['vdim'])
+            w[pre + 'mix.a1'] = matrix(decay_rank, width, 2.0)
+            w[pre + 'mix.a2'] = matrix(hd, decay_rank, 2.0)
+            w[pre + 'mix.a2.b'] = (decay_bias + torch.randn(hd, generator=g)).to(torch.bfloat16).to(torch.float64)
+        f = layer['mlp']
+        if f is not None:
+            r = f['router']
+            w[pre + 'norm2'], w[pre + 'norm2b'] = scale(width), scale(width)
+            w[pre + 'mlp.router'] = matrix(r['experts'] + r['identity'], width, 3.0)
+            w[pre + 'mlp.correction'] = (0.2 * torch.randn(r['experts'] + r['identity'], generator=g)).to(torch.bfloat16).to(torch.float64)
+            for e in range(r['experts']):
+                w[f'{pre}mlp.e{e}.gate'] = matrix(f['expert']['ff'], width, 1.5)
+                w[f'{pre}mlp.e{e}.up'] = matrix(f['expert']['ff'], width, 1.5)
+                w[f'{pre}mlp.e{e}.down'] = matrix(width, f['expert']['ff'])
+    return w

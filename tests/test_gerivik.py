@@ -1,0 +1,457 @@
+"""The Gerivik design in the engine against its plain whole-sequence restatement (``plain_gerivik``), under every way
+of cutting the work: whole prompts, token-by-token decoding, portions down to two tokens, unequal batches, pages and
+state slots that are freed and used again, and generation through the serving loop; then each mechanism alone, with
+weights or inputs made so that a fault shows (a far key that decides the answer, a soft cap that saturates, a router
+whose groups and correction decide the choice, identity experts, decays near 0 and near 1).
+
+Each model test runs three ways, as the step function's own tests do: on the CPU with the kernels' plain references
+substituted, and on the GPU with the HIP kernels in float32 and in bfloat16 (marked ``gpu``).  Page and state storage
+is filled with NaN first.  Configurations are small and their sizes differ from one another in every field.
+"""
+import json
+import math
+import random
+
+import pytest
+import torch
+
+import plain_gerivik as plain
+from conftest import write_model_folder
+from qil_amd.engine import ModelRunner, StepEntry
+from qil_amd.weights import load_model
+
+BACKENDS = [pytest.param(('cpu', torch.float32), id='cpu-refs'),
+            pytest.param(('cuda', torch.float32), id='gpu-f32', marks=pytest.mark.gpu),
+            pytest.param(('cuda', torch.bfloat16), id='gpu-bf16', marks=pytest.mark.gpu)]
+
+
+def _mixed():
+    layers = [
+        plain.gla_layer(heads=2, dim=24, vdim=40, tau=6.0,
+                        mlp=plain.moe_mlp(ff=40, limit=1.5, experts=6, identity=2, top=3, count=4, keep=2)),
+        plain.attention_layer(heads=6, kv_heads=2, dim=16, vdim=24, rot_dims=8, scale=0.4, softcap=3.0, base=500.0,
+                              mlp=plain.moe_mlp(ff=24, limit=0.75, experts=5, identity=0, top=2)),
+        plain.gla_layer(heads=3, dim=16, vdim=16, tau=20.0),
+    ]
+    layers += [plain.shared(layers, 1), plain.shared(layers, 0)]
+    return plain.make_config(layers, vocab=97, width=48, scale=5.0)
+
+
+def _wide():
+    # state columns beyond one wave (80, 130), key sizes that are no powers of two, values wider than keys and the
+    # other way round, every head its own key/value head, one key/value head for all
+    layers = [
+        plain.gla_layer(heads=2, dim=72, vdim=130, tau=3.0, mlp=plain.moe_mlp(ff=56, limit=3.0, experts=3, identity=1, top=1)),
+        plain.attention_layer(heads=5, kv_heads=5, dim=12, vdim=10, rot_dims=12, scale=1.0, softcap=30.0,
+                              mlp=plain.moe_mlp(ff=20, limit=1.0, experts=9, identity=3, top=4, count=3, keep=3)),
+        plain.attention_layer(heads=4, kv_heads=1, dim=20, vdim=36, rot_dims=2, scale=0.05, softcap=0.5, base=3.0),
+        plain.gla_layer(heads=1, dim=40, vdim=80, tau=1.0),
+    ]
+    layers.insert(2, plain.shared(layers, 0))
+    return plain.make_config(layers, vocab=61, width=40, scale=0.7, eps=1e-5)
+
+
+def _attention():
+    layers = [plain.attention_layer(heads=4, kv_heads=2, dim=24, vdim=24, rot_dims=16, scale=24 ** -0.5, softcap=8.0,
+                                    mlp=plain.moe_mlp(ff=48, limit=2.5, experts=4, identity=4, top=2, count=2, keep=1))]
+    layers.append(plain.shared(layers, 0))
+    return plain.make_config(layers, vocab=50, width=32, scale=2.0)
+
+
+# (configuration, seed, page size, spread of the matrices)
+CONFIGS = {'mixed': (_mixed(), 11, 8, 1.0), 'wide': (_wide(), 12, 16, 1.0), 'attention': (_attention(), 13, 4, 1.5)}
+
+
+def tokens_for(config, length, seed):
+    r = random.Random(seed)
+    return [r.randrange(config['vocab']) for _ in range(length)]
+
+
+def error(actual, expected):
+    """The largest row error: root mean square over the vocabulary of the difference (its mean taken off), over the
+    root mean square of the expected logits."""
+    difference = actual.double().cpu() - expected.double()
+    difference = difference - difference.mean(dim=-1, keepdim=True)
+    return (difference.square().mean(dim=-1).sqrt() / expected.double().square().mean().sqrt()).max().item()
+
+
+# The engine in float32 is 1e-6 to 2e-5 from the float64 plain model on these configurations; in bfloat16 (activations
+# between kernels rounded; state, decays, scores, norms, router and residual sums float32) 0.01 to 0.05.  A sequence
+# that loses its context half way (a lost state, another request's pages) is 0.1 to 0.7 away.
+LIMIT = {torch.float32: 1e-4, torch.bfloat16: 0.07}
+
+
+class Case:
+    def __init__(self, name, config, weights, model, page_size, dtype):
+        self.name, self.config, self.weights, self.model, self.page_size, self.dtype = name, config, weights, model, page_size, dtype
+        self._expected = {}
+
+    def expected(self, tokens):
+        key = tuple(tokens)
+        if key not in self._expected:
+            self._expected[key] = plain.logits(tokens, self.weights, self.config)
+        return self._expected[key]
+
+    def runner(self, pages, requests=4, graphs=False):
+        runner = ModelRunner(self.model, num_pages=pages, page_size=self.page_size, max_requests=requests, graphs=graphs)
+        for group in runner.cache.kv_groups:
+            for tensor in ([group['k'], group['v']] if 'k' in group else group['tensors'].values()):
+                tensor.fill_(float('nan'))
+        for group in runner.cache.state_groups:
+            group['state'].fill_(float('nan'))
+        return runner
+
+    def close(self, actual, expected, what='', slack=1.0):
+        assert torch.isfinite(actual).all(), what
+        e = error(actual, expected)
+        assert e <= LIMIT[self.dtype] * slack, f'{what}: error {e:.3e} ({self.dtype})'
+
+
+@pytest.fixture(params=BACKENDS)
+def backend(request):
+    device, dtype = request.param
+    if device == 'cpu':
+        request.getfixturevalue('cpu_kernels')
+    return device, dtype
+
+
+def make_case(name, config, weights, backend, folder, page_size):
+    device, dtype = backend
+    write_model_folder(folder, config, weights, torch.bfloat16)
+    return Case(name, config, weights, load_model(folder, dtype=dtype, device=device), page_size, dtype)
+
+
+@pytest.fixture(params=sorted(CONFIGS))
+def case(request, backend, tmp_path):
+    config, seed, page_size, spread = CONFIGS[request.param]
+    return make_case(request.param, config, plain.random_weights(config, seed, spread), backend, tmp_path / request.param, page_size)
+
+
+def feed(runner, name, tokens, cuts):
+    """One request alone, its tokens in steps of the given sizes (the rest one by one); the logits of every place."""
+    runner.admit(name)
+    rows, at, sizes = [], 0, list(cuts)
+    while at < len(tokens):
+        size = min(sizes.pop(0) if sizes else 1, len(tokens) - at)
+        rows.append(runner.step([StepEntry(name, tuple(tokens[at:at + size]), tuple(range(size)))]))
+        at += size
+    runner.release(name)
+    return torch.cat(rows)
+
+
+# ------------------------------------------------------------------------------------------------ whole models
+def test_whole_prompts(case):
+    runner = case.runner(pages=64)
+    for length, seed in ((1, 1), (2, 2), (37, 3), (150, 4)):
+        tokens = tokens_for(case.config, length, seed)
+        case.close(feed(runner, 'r', tokens, [length]), case.expected(tokens), f'{length} tokens')
+    runner.cache.check()
+
+
+def test_decoding_token_by_token_equals_the_prompt(case):
+    """The first tokens of a sequence one by one, then a long run of single tokens behind a prompt."""
+    runner = case.runner(pages=64)
+    tokens = tokens_for(case.config, 45, 5)
+    case.close(feed(runner, 'r', tokens, []), case.expected(tokens), 'one by one from the first token')
+    tokens = tokens_for(case.config, 140, 6)
+    case.close(feed(runner, 'r', tokens, [50]), case.expected(tokens), '50, then 90 single tokens')
+
+
+def test_decode_graphs_replay_the_same_logits(case):
+    if case.model.device.type != 'cuda':
+        pytest.skip('graphs are a GPU matter')
+    runner = case.runner(pages=64, graphs=True)
+    tokens = tokens_for(case.config, 70, 7)
+    case.close(feed(runner, 'r', tokens, [20]), case.expected(tokens), 'decode steps from graphs')
+    assert runner.graphs.safe() and runner.graphs.replays >= 20
+
+
+@pytest.mark.parametrize('cuts', [[2] * 40, [3, 2, 17, 2, 5, 31, 2, 2, 9], [16, 16, 1, 15, 33, 7], [63, 2, 1, 1, 2],
+                                  [64, 64, 65, 2], [130, 31, 33]])
+def test_portions_of_changing_size(case, cuts):
+    """Portions down to two tokens, cut inside pages and at their borders and at the edges of the recurrence's blocks of
+    64 tokens (portions of 32 tokens and more run in such blocks, shorter ones token by token); the rest one by one."""
+    runner = case.runner(pages=64)
+    tokens = tokens_for(case.config, max(90, sum(cuts) + 3), 8)
+    case.close(feed(runner, 'r', tokens, cuts), case.expected(tokens), f'cuts {cuts[:6]}')
+
+
+def test_unequal_requests_together_and_slots_used_again(case):
+    """Up to three live requests of unequal lengths, portions beside single tokens; requests end and others take their
+    pages and state slots (three slots, six requests); some steps leave a live request out."""
+    lengths = dict(a=71, b=9, c=38, d=1, e=55, f=20)
+    sequences = {name: tokens_for(case.config, n, 20 + i) for i, (name, n) in enumerate(lengths.items())}
+    pages = -(-(71 + 55 + 38) // case.page_size) + 3
+    runner = case.runner(pages=pages, requests=3)
+    waiting, live = list(sequences), []
+    fed = {name: 0 for name in sequences}
+    got = {name: [] for name in sequences}
+    r = random.Random(3)
+    used_slots = []
+    while waiting or live:
+        while waiting and len(live) < 3:
+            name = waiting.pop(0)
+            assert runner.admit(name)
+            used_slots.append(runner.cache.slots[name])
+            live.append(name)
+        entries = []
+        for name in live:
+            if len(live) > 1 and r.random() < 0.2:
+                continue                                      # left out of this step
+            left = len(sequences[name]) - fed[name]
+            size = min(left, r.choice([1, 1, 2, 3, 7, 16, 29, 40]))
+            entries.append(StepEntry(name, tuple(sequences[name][fed[name]:fed[name] + size]), tuple(range(size))))
+        if not entries:
+            continue
+        logits = runner.step(entries)
+        at = 0
+        for entry in entries:
+            size = len(entry.tokens)
+            got[entry.request].append(logits[at:at + size])
+            at += size
+            fed[entry.request] += size
+            if fed[entry.request] == len(sequences[entry.request]):
+                runner.release(entry.request)
+                live.remove(entry.request)
+        runner.cache.check()
+    assert sorted(set(used_slots)) == [0, 1, 2] and len(used_slots) == 6
+    assert runner.cache.free_pages == [pages] * len(runner.cache.kv_groups)
+    for name, tokens in sequences.items():
+        case.close(torch.cat(got[name]), case.expected(tokens), f'request {name}')
+
+
+def test_a_batch_changes_nothing(case):
+    """The same request alone and beside others gives the same logits (beyond rounding: the same kernels may split
+    their sums differently)."""
+    a, b, c = (tokens_for(case.config, n, 40 + n) for n in (33, 12, 50))
+    alone = feed(case.runner(pages=32), 'a', a, [20, 2])
+    runner = case.runner(pages=32)
+    for name in 'abc':
+        runner.admit(name)
+    rows = [runner.step([StepEntry('b', tuple(b[:5])), StepEntry('a', tuple(a[:20]), tuple(range(20))), StepEntry('c', tuple(c[:31]))])]
+    rows.append(runner.step([StepEntry('a', tuple(a[20:22]), (0, 1)), StepEntry('c', tuple(c[31:32])), StepEntry('b', tuple(b[5:]))])[:2])
+    for i in range(22, 33):
+        rows.append(runner.step([StepEntry('c', (c[i + 10],)), StepEntry('a', (a[i],), (0,))]))
+    together = torch.cat(rows)
+    assert error(together, alone.cpu()) <= LIMIT[case.dtype] / 2
+    case.close(together, case.expected(a), 'beside others')
+
+
+def test_generation_through_the_serving_loop(case):
+    """Greedy generation by the engine's own entry point and scheduler: every drawn token is (within the dtype's
+    rounding) the best one of the plain logits of the engine's own sequence so far."""
+    from qil_amd.engine import Engine
+    prompts = [tokens_for(case.config, n, 60 + n) for n in (5, 1, 23, 12, 9)]
+    engine = Engine(case.model, num_pages=24, page_size=case.page_size, token_budget=20, prefill_chunk=7, max_active=3)
+    reports = engine.generate(prompts, max_new_tokens=12, ignore_eos=True)
+    engine.cache.check()
+    assert engine.cache.free_pages == [24] * len(engine.cache.kv_groups)
+    slack = 1e-4 if case.dtype == torch.float32 else 0.06
+    for prompt, report in zip(prompts, reports):
+        output = report['token_ids']
+        assert len(output) == 12 and report['finish_reason'] == 'length'
+        rows = plain.logits(prompt + output, case.weights, case.config)
+        spread = rows.std().item()
+        for index, token in enumerate(output):
+            row = rows[len(prompt) + index - 1]
+            assert row[token] >= row.max() - slack * spread, f'token {index} of {prompt}'
+    if case.dtype == torch.float32:
+        assert [r['token_ids'] for r in reports][0] == plain.greedy(prompts[0], 12, case.weights, case.config)
+
+
+# ------------------------------------------------------------------------------------------------ each mechanism alone
+ALONE = {
+    'attention-one-head': plain.make_config(
+        [plain.attention_layer(heads=1, kv_heads=1, dim=10, vdim=14, rot_dims=2, scale=0.9, softcap=2.0)], vocab=40, width=24),
+    'attention-values-narrower': plain.make_config(
+        [plain.attention_layer(heads=9, kv_heads=3, dim=36, vdim=4, rot_dims=36, scale=0.02, softcap=100.0, base=20.0)],
+        vocab=40, width=36, scale=9.0),
+    'memory': plain.make_config([plain.gla_layer(heads=3, dim=10, vdim=70, tau=2.0)], vocab=40, width=30, scale=0.3),
+    'memory-one-head-long-keys': plain.make_config([plain.gla_layer(heads=1, dim=130, vdim=12, tau=64.0)], vocab=40, width=20),
+    'memory-twice': plain.make_config([plain.gla_layer(heads=2, dim=8, vdim=8, tau=1.5), dict(plain.gla_layer(heads=2, dim=8, vdim=8, tau=1.5), weights_of=0)],
+                                      vocab=40, width=16),
+    'experts-every-one-chosen': plain.make_config(
+        [plain.gla_layer(heads=1, dim=8, vdim=8, tau=4.0, mlp=plain.moe_mlp(ff=18, limit=0.5, experts=3, identity=0, top=3))],
+        vocab=40, width=28),
+    'experts-one-of-many-groups': plain.make_config(
+        [plain.gla_layer(heads=1, dim=8, vdim=8, tau=4.0,
+                         mlp=plain.moe_mlp(ff=10, limit=4.0, experts=13, identity=7, top=1, count=10, keep=1))],
+        vocab=40, width=24),
+    'experts-identity-only-group': plain.make_config(
+        [plain.attention_layer(heads=2, kv_heads=1, dim=8, vdim=8, rot_dims=4, scale=0.5, softcap=10.0,
+                               mlp=plain.moe_mlp(ff=33, limit=1.0, experts=4, identity=4, top=3, count=2, keep=2))],
+        vocab=40, width=20),
+}
+
+
+@pytest.mark.parametrize('name', sorted(ALONE))
+def test_each_mechanism_alone(name, backend, tmp_path):
+    """Models of one layer: one mechanism each, at sizes where fields that often coincide differ (key size and value
+    size, heads and key/value heads, rotated part and head) and where counts are 1."""
+    config = ALONE[name]
+    case = make_case(name, config, plain.random_weights(config, 5, 1.5, decay_rank=3), backend, tmp_path / name, 8)
+    tokens = tokens_for(config, 100, 9)
+    runner = case.runner(pages=16)
+    case.close(feed(runner, 'r', tokens, [100]), case.expected(tokens), 'whole')
+    case.close(feed(runner, 'r', tokens, [13, 2, 9, 8, 40]), case.expected(tokens), 'portions, then single tokens')
+
+
+def test_a_far_key_decides(backend, tmp_path):
+    """One key hundreds of tokens back, at a page's last place, is the only one a late query likes: its value must
+    come through, in a prompt, in portions and in decoding.  The marked token's input excites one channel and the asking
+    token's another, and the query matrix's column for the second is the key matrix's column for the first: the asking
+    query is the marked key (both of root mean square 1 after the norm), a score of dim * scale against about a third of
+    that for the best of the other keys."""
+    config = plain.make_config([plain.attention_layer(heads=2, kv_heads=1, dim=32, vdim=8, rot_dims=2, scale=1.0,
+                                                      softcap=60.0, base=1e6)], vocab=12, width=48)
+    w = plain.random_weights(config, 3, 1.0)
+    embed = w['embed'].clone()
+    embed[10], embed[11] = 0.0, 0.0
+    embed[10, 5], embed[11, 7] = 8.0, 8.0
+    w['embed'] = embed
+    w['l0.norm1'] = torch.ones(48, dtype=torch.float64)
+    query = w['l0.mix.q'].clone()
+    query[:32, 7], query[32:, 7] = w['l0.mix.k'][:, 5], w['l0.mix.k'][:, 5]
+    w['l0.mix.q'] = query
+    case = make_case('far', config, w, backend, tmp_path / 'far', 16)
+    tokens = [t % 10 for t in tokens_for(config, 420, 2)]
+    tokens[15] = 10                                   # the last place of the first page
+    asking = [300, 401, 419]
+    for place in asking:
+        tokens[place] = 11
+    expected = case.expected(tokens)
+    other = list(tokens)
+    other[15] = 3
+    moved = error(plain.logits(other, w, config)[asking], expected[asking])
+    assert moved > 0.05, 'the test lost its point: the far key does not matter'
+    runner = case.runner(pages=40)
+    case.close(feed(runner, 'r', tokens, [420])[asking], expected[asking], 'in a prompt')
+    case.close(feed(runner, 'r', tokens, [128, 130, 100, 42])[asking], expected[asking], 'in portions')
+    case.close(feed(runner, 'r', tokens, [400])[asking[1:]], expected[asking[1:]], 'decoded')
+
+
+def test_the_cap_saturates_and_an_old_memory_fades(backend, tmp_path):
+    """Scores far beyond the cap (all keys then weigh almost alike, which an uncapped softmax would not give), and a
+    memory whose decays run from almost 0 to almost 1: the plain model decides."""
+    layers = [plain.attention_layer(heads=2, kv_heads=2, dim=8, vdim=8, rot_dims=4, scale=25.0, softcap=0.25),
+              plain.gla_layer(heads=2, dim=8, vdim=8, tau=0.5)]
+    config = plain.make_config(layers, vocab=30, width=16, scale=2.0)
+    w = plain.random_weights(config, 8, 1.0, decay_bias=0.0)
+    w['l1.mix.a2.b'] = torch.linspace(-9.0, 9.0, 16, dtype=torch.float64).to(torch.bfloat16).to(torch.float64)
+    uncapped = json.loads(json.dumps(config))
+    uncapped['layers'][0]['mixer']['softcap'] = 1e6
+    tokens = tokens_for(config, 150, 4)
+    assert error(plain.logits(tokens, w, uncapped), plain.logits(tokens, w, config)) > 0.05
+    case = make_case('cap', config, w, backend, tmp_path / 'cap', 8)
+    runner = case.runner(pages=24)
+    case.close(feed(runner, 'r', tokens, [150]), case.expected(tokens), 'whole')
+    case.close(feed(runner, 'r', tokens, [70, 3, 37]), case.expected(tokens), 'portions and single tokens')
+
+
+# ------------------------------------------------------------------------------------------------ the router's rules
+def test_the_router_follows_groups_correction_and_identity():
+    """The plain router on scores made by hand: the correction changes the choice and not the weights; a group is
+    judged by its best corrected score; experts outside the kept groups are out however good; weights are the plain
+    softmax scores, not renormalised; identity experts pass their input."""
+    width, r = 8, dict(experts=4, identity=2, top=2, groups=dict(count=3, keep=2))
+    logit = torch.tensor([2.0, 0.0, 1.9, 1.8, 0.5, 0.4], dtype=torch.float64)
+    h = torch.zeros(1, width, dtype=torch.float64)
+    h[0, 0] = 1.0
+    router = torch.zeros(6, width, dtype=torch.float64)
+    router[:, 0] = logit
+    w = {'router': router, 'correction': torch.zeros(6, dtype=torch.float64)}
+    s = torch.softmax(logit, dim=0)
+    chosen, weights = plain.route(h, w, '', r)
+    assert chosen.tolist() == [[0, 2]] and torch.allclose(weights[0], s[[0, 2]])      # groups (0,1) and (2,3) are kept
+    w['correction'] = torch.tensor([0.0, 0.0, 0.0, 0.0, 0.9, 0.0], dtype=torch.float64)
+    chosen, weights = plain.route(h, w, '', r)                                        # group (4,5) now leads, (2,3) is out
+    assert chosen.tolist() == [[4, 0]] and torch.allclose(weights[0], s[[4, 0]]) and weights.sum() < 0.9
+    w['correction'] = torch.tensor([-5.0, -5.0, -5.0, -5.0, -5.0, -5.1], dtype=torch.float64)
+    chosen, _ = plain.route(h, w, '', r)                                              # negative choice scores: out means -inf, not 0
+    assert chosen.tolist() == [[0, 2]]
+    f = dict(expert=dict(ff=4, limit=1.0), router=dict(experts=0, identity=6, top=2, groups=dict(count=3, keep=2)))
+    w['correction'] = torch.zeros(6, dtype=torch.float64)
+    assert torch.allclose(plain.moe(h, w, '', f), h * (s[0] + s[2]))
+
+
+def test_the_plain_model_cuts_like_its_parts():
+    """The oracle itself: a prefix's logits do not depend on what follows (every mixer is causal), and a layer that
+    uses another's tensors is one more run of it."""
+    config, seed, _, spread = CONFIGS['mixed']
+    weights = plain.random_weights(config, seed, spread)
+    tokens = tokens_for(config, 30, 1)
+    whole, streams = plain.logits(tokens, weights, config), []
+    prefix = plain.logits(tokens[:17], weights, config, streams=streams)
+    assert torch.allclose(whole[:17], prefix, atol=1e-9) and len(streams) == 5
+    unrolled = json.loads(json.dumps(config))
+    copied = dict(weights)
+    for index, layer in enumerate(unrolled['layers']):
+        source = layer.pop('weights_of', None)
+        if source is not None:
+            copied.update({name.replace(f'l{source}.', f'l{index}.', 1): t for name, t in weights.items() if name.startswith(f'l{source}.')})
+    assert torch.allclose(plain.logits(tokens, copied, unrolled), whole, atol=1e-12)
+
+
+def test_config_round_trip_and_refusals():
+    from qil_amd.config import ConfigError, GerivikConfig
+    from qil_amd.registry import architecture_for
+    config = CONFIGS['mixed'][0]
+    typed = GerivikConfig.from_dict(config)
+    assert architecture_for(config).name == 'Gerivik'
+    assert [typed.weights_layer(i) for i in range(5)] == [0, 1, 2, 1, 0]
+    assert GerivikConfig.from_dict(json.loads(json.dumps(typed.to_dict()))) == typed
+    layers = config['layers']
+
+    def with_mixer(index, **changes):
+        return dict(layers[index], mixer=dict(layers[index]['mixer'], **changes))
+
+    for broken in (dict(config, window=4), dict(config, embedding=dict(scale=0)), dict(config, norm=dict(eps=1e-6, kind='layer')),
+                   dict(config, layers=[dict(layers[0], type='conv')]),
+                   dict(config, layers=[with_mixer(1, window=3)]), dict(config, layers=[with_mixer(1, kv_heads=4)]),
+                   dict(config, layers=[with_mixer(1, rot=dict(base=10.0, dims=18))]), dict(config, layers=[with_mixer(0, tau=0)]),
+                   dict(config, layers=[dict(layers[0], weights_of=0)]),
+                   dict(config, layers=[layers[0], dict(layers[1], weights_of=0)]),
+                   dict(config, layers=layers[:4] + [dict(layers[1], weights_of=3)]),
+                   dict(config, layers=[dict(layers[0], mlp=plain.moe_mlp(ff=8, limit=1.0, experts=5, identity=2, top=2, count=2, keep=1))]),
+                   dict(config, layers=[dict(layers[0], mlp=plain.moe_mlp(ff=8, limit=1.0, experts=4, identity=2, top=4, count=3, keep=1))])):
+        with pytest.raises(ConfigError):
+            GerivikConfig.from_dict(broken)
+
+
+def test_the_decay_rank_comes_from_the_tensors(tmp_path, cpu_kernels):
+    """No key of the configuration gives the inner size of the decay's low-rank product: models whose tensors differ
+    there load and run, and tensors that do not fit each other are refused."""
+    config = ALONE['memory']
+    for rank in (1, 7):
+        weights = plain.random_weights(config, 2, decay_rank=rank)
+        case = make_case(f'rank{rank}', config, weights, ('cpu', torch.float32), tmp_path / f'rank{rank}', 8)
+        tokens = tokens_for(config, 20, rank)
+        case.close(feed(case.runner(pages=8), 'r', tokens, [20]), case.expected(tokens), f'rank {rank}')
+    weights['l0.mix.a1'] = weights['l0.mix.a1'][:5]
+    write_model_folder(tmp_path / 'torn', config, weights, torch.bfloat16)
+    with pytest.raises(ValueError):
+        load_model(tmp_path / 'torn', dtype=torch.float32, device='cpu')
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
+def test_trace_replay_program(tmp_path, dtype):
+    """``bin/trace_run`` on a Gerivik folder: requests alone and whole, their last tokens one by one, portions down to
+    two tokens, and up to four live requests in a pool of pages and state slots that is used again."""
+    from test_engine_gpu import collect, replay, traces
+    config, seed, _, spread = CONFIGS['mixed']
+    weights = plain.random_weights(config, seed, spread)
+    folder = write_model_folder(tmp_path / 'model', config, weights, torch.bfloat16)
+    prompts, shapes = traces(dict(vocab_size=config['vocab']), seed)
+    expected = {request: plain.logits(tokens, weights, config) for request, tokens in prompts.items()}
+    limit = LIMIT[getattr(torch, dtype)]
+    for shape, (steps, max_tokens) in shapes.items():
+        out = tmp_path / shape
+        replay(folder, dtype, steps, out, max_tokens)
+        rows = collect(out, steps, config['vocab'])
+        assert rows, shape
+        for request, items in rows.items():
+            got = torch.stack([row for _, row in items])
+            assert torch.isfinite(got).all()
+            e = error(got, expected[request][[position for position, _ in items]])
+            assert e <= limit, f'{shape} {request}: error {e:.3e}'
