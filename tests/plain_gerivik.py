@@ -94,6 +94,27 @@ def route(h, w, pre, r):
     return chosen, s.gather(1, chosen)
 
 
+def route_margin(h, w, pre, r):
+    """How far every token's choice is from another one [T]: the smaller of the gap between the last kept and the
+    first dropped group and the gap between the last chosen and the first unchosen output.  Tests leave out tokens
+    whose margin is within rounding: there the choice is not the design's to decide."""
+    s = torch.softmax(h @ w[pre + 'router'].t(), dim=-1)
+    choice = s + w[pre + 'correction']
+    total = r['experts'] + r['identity']
+    count, keep = r['groups']['count'], r['groups']['keep']
+    best = choice.reshape(-1, count, total // count).max(dim=-1).values
+    margin = torch.full((h.shape[0],), math.inf, dtype=h.dtype)
+    if keep < count:
+        ordered = best.sort(dim=-1, descending=True).values
+        margin = ordered[:, keep - 1] - ordered[:, keep]
+    kept = torch.zeros_like(best, dtype=torch.bool)
+    kept.scatter_(1, best.topk(keep, dim=-1).indices, True)
+    ordered = choice.masked_fill(~kept.repeat_interleave(total // count, dim=1), -math.inf).sort(dim=-1, descending=True).values
+    if r['top'] < total:
+        margin = torch.minimum(margin, ordered[:, r['top'] - 1] - ordered[:, r['top']])
+    return margin
+
+
 def moe(h, w, pre, f):
     r = f['router']
     chosen, weights = route(h, w, pre, r)
@@ -108,8 +129,9 @@ def moe(h, w, pre, f):
 
 
 # ---------------------------------------------------------------------------------------------- the model
-def logits(tokens, weights, config, dtype=torch.float64, streams=None):
-    """Logits [T, vocab] of one sequence.  ``streams``: a list that receives the residual stream after every layer run."""
+def logits(tokens, weights, config, dtype=torch.float64, streams=None, margins=None):
+    """Logits [T, vocab] of one sequence.  ``streams``: a list that receives the residual stream after every layer run;
+    ``margins``: a list that receives every routed feed-forward's ``route_margin``."""
     w = {name: t.to(dtype) for name, t in weights.items()}
     eps = config['norm']['eps']
     positions = torch.arange(len(tokens))
@@ -123,6 +145,8 @@ def logits(tokens, weights, config, dtype=torch.float64, streams=None):
             mixed = gla(h, w, pre + 'mix.', layer['mixer'], eps)
         x = x + rms_norm(mixed, w[pre + 'norm1b'], eps)
         if layer['mlp'] is not None:
+            if margins is not None:
+                margins.append(route_margin(rms_norm(x, w[pre + 'norm2'], eps), w, pre + 'mlp.', layer['mlp']['router']))
             fed = moe(rms_norm(x, w[pre + 'norm2'], eps), w, pre + 'mlp.', layer['mlp'])
             x = x + rms_norm(fed, w[pre + 'norm2b'], eps)
         if streams is not None:
