@@ -222,22 +222,44 @@ def fubapel_config(z, layers, vocab):
                 loop=dict(start=0, stop=0, times=1), norm=dict(eps=1e-5), residual_mult=1.0)
 
 
+def gerivik_config(z, layers, vocab):
+    """`layers` layers in turns of gated linear attention and capped attention, a routed feed-forward behind each: 30
+    experts and 2 identity experts in 4 groups of which 2 are kept, 4 chosen, every expert a quarter of the dense
+    feed-forward (a token's experts together are as large as the dense one)."""
+    ffn = dict(kind='moe', expert=dict(ff=z['ff'] // 4, limit=7.0),
+               router=dict(experts=30, identity=2, top=4, groups=dict(count=4, keep=2)))
+    kinds = [
+        dict(type='gla', mlp=ffn, mixer=dict(heads=z['memory_heads'], dim=z['memory_dim'], vdim=z['memory_vdim'], tau=16.0)),
+        dict(type='attention', mlp=ffn,
+             mixer=dict(heads=z['heads'], kv_heads=max(1, z['heads'] // 4), dim=z['dim'], vdim=z['dim'],
+                        rot=dict(base=10000.0, dims=z['rot_dim']), scale=z['dim'] ** -0.5, softcap=50.0)),
+    ]
+    return dict(architecture='Gerivik', vocab=vocab, width=z['width'], embedding=dict(scale=1.0),
+                layers=[kinds[i % 2] for i in range(layers)], norm=dict(eps=1e-6))
+
+
 def designs_phase(args, torch, dtype):
-    """Prefill tokens a second and decode milliseconds a step of Fubapel models whose layers are all of one kind (and of
-    the three kinds in turns), beside dense Qwen3 of the same width, feed-forward, depth and attention heads."""
+    """Prefill tokens a second and decode milliseconds a step of a design's models whose layers are all of one kind
+    (and of its kinds in turns), beside dense Qwen3 of the same width, feed-forward, depth and attention heads."""
     from qil_amd import Engine, Qwen3
     from qil_amd.engine import ModelRunner, StepEntry
     z, layers, vocab, page_size = DESIGN_SIZES[args.design_sizes], args.layers or 6, 32768, 16
     generator = torch.Generator().manual_seed(99)
-    mixed = fubapel_config(z, layers, vocab)
-    models = {'fubapel (kinds in turns)': mixed}
-    for index, name in enumerate(('latent attention', 'gated memory', 'decaying memory')):
-        models[f'fubapel ({name} only)'] = dict(mixed, layers=[mixed['layers'][index]] * layers)
+    if args.design == 'gerivik':
+        mixed = gerivik_config(z, layers, vocab)
+        models = {'gerivik (kinds in turns)': mixed}
+        for index, name in enumerate(('gated linear attention', 'capped attention')):
+            models[f'gerivik ({name} only)'] = dict(mixed, layers=[mixed['layers'][index]] * layers)
+    else:
+        mixed = fubapel_config(z, layers, vocab)
+        models = {'fubapel (kinds in turns)': mixed}
+        for index, name in enumerate(('latent attention', 'gated memory', 'decaying memory')):
+            models[f'fubapel ({name} only)'] = dict(mixed, layers=[mixed['layers'][index]] * layers)
     models['qwen3 (equal sizes)'] = dict(SIZES, vocab_size=vocab, hidden_size=z['width'], intermediate_size=z['ff'],
                                          num_hidden_layers=layers, num_attention_heads=z['heads'],
                                          num_key_value_heads=max(1, z['heads'] // 4), head_dim=z['dim'],
                                          max_position_embeddings=max(args.history + args.steps + args.warmup + 64, args.prefill_tokens))
-    report = {'phase': 'designs', 'sizes': args.design_sizes, 'layers': layers, 'dtype': args.dtype,
+    report = {'phase': 'designs', 'design': args.design, 'sizes': args.design_sizes, 'layers': layers, 'dtype': args.dtype,
               'prefill_tokens': args.prefill_tokens, 'batch': args.batch, 'history': args.history, 'models': {}}
     for name, config in models.items():
         model = Qwen3.from_config(config, seed=0, dtype=dtype, device='cuda:0', on_device=True)
@@ -301,7 +323,8 @@ def main():
                              'mixed: steps of one prompt portion (--portion tokens) beside --batch decoded rows.  attention: the '
                              'attention kernels alone, at the reference\'s own shapes and at the benchmark\'s.  products: a layer\'s '
                              'matrix products at --prefill-tokens rows alone, GPU BLAS against own kernel.  designs: prefill and decode of the '
-                             'Fubapel design at --design-sizes beside dense Qwen3 of equal sizes (--layers, default 6)')
+                             'design named by --design at --design-sizes beside dense Qwen3 of equal sizes (--layers, default 6)')
+    parser.add_argument('--design', default='fubapel', choices=['fubapel', 'gerivik'], help='the design of --phase designs')
     parser.add_argument('--design-sizes', default='1b', choices=sorted(DESIGN_SIZES), help='layer sizes of --phase designs')
     parser.add_argument('--portion', type=int, default=128, help='tokens of the prompt portion of a mixed step')
     parser.add_argument('--own-products', action='store_true',

@@ -49,14 +49,18 @@ __device__ __forceinline__ int prompt_row(int kl) {
 // group hands its sums over in LDS and the first adds them to its own.  For prompts so short that blocks of 4 waves
 // are fewer than the CUs: every SIMD then has two waves.  (It does not help longer prompts: a wave-tile takes 1.75 us
 // of its SIMD's issue slots whether the wave is alone there or not, and 2,048 tokens are 33 wave-tiles a SIMD.)
-template <int WAVES, bool SPLIT = false>
+// CAP: scores are scaled and capped softly (softcap * tanh(score / softcap)) as they leave the matrix cores; the
+// exponent then scales nothing.
+template <int WAVES, bool SPLIT = false, bool CAP = false>
 __global__ void __launch_bounds__(WAVES * QIL_WAVE, WAVES == 4 ? 2 : 1)
 attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_cache,
                    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_tables, int table_stride,
                    const int* __restrict__ cu_seqlens, const int* __restrict__ seq_starts, bf16_t* __restrict__ out,
                    int heads, int kv_heads, int page_size, int window, float scale, int GH, int chunks, int ps_shift,
                    float* __restrict__ part_acc, float* __restrict__ part_m, float* __restrict__ part_l, int P,
-                   int parts) {
+                   int parts, float softcap) {
+  const float raw_scale = scale;
+  if (CAP) scale = 1.f;
   constexpr int D = PROMPT_D, BK = PROMPT_BK, THREADS = WAVES * QIL_WAVE;
   constexpr int GW = SPLIT ? WAVES / 2 : WAVES;            // waves that share a tile of keys
   constexpr int WFRAGS = D / 16, WTILES = D / 32;
@@ -245,6 +249,13 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
       if (ks == 2 * LOADS - 1) held = look_up(k0 + 2 * BK);
       __builtin_amdgcn_sched_barrier(0);
     }
+    if (CAP) {
+      const float fast = 2.88539008177793f / softcap;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s[kt][i] = soft_cap_fast(s[kt][i] * raw_scale, softcap, fast);
+    }
     if (masked) {                                          // keys a row does not see get score -inf (probability 0)
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
@@ -423,15 +434,15 @@ attn_prompt_kernel(const bf16_t* __restrict__ q, int q_stride, const bf16_t* __r
           make_uint2(pack_bf16(ow[t][4 * j] * inv, ow[t][4 * j + 1] * inv), pack_bf16(ow[t][4 * j + 2] * inv, ow[t][4 * j + 3] * inv));
 }
 
-template <int WAVES, bool SPLIT = false>
+template <int WAVES, bool SPLIT = false, bool CAP = false>
 static int launch_prompt(const void* q, int q_stride, const void* k_cache, const void* v_cache, const int* block_tables,
                          int table_stride, const int* cu_seqlens, const int* seq_starts, void* out, int n_seqs,
                          int max_query, int heads, int kv_heads, int page_size, int window, float scale, hipStream_t s,
-                         float* workspace, int total_rows, int P, int parts) {
+                         float* workspace, int total_rows, int P, int parts, float softcap = 0.f) {
   const int g = heads / kv_heads;
   const int GH = g >= 3 ? 4 : g, chunks = (g + GH - 1) / GH, RT = (SPLIT ? WAVES / 2 : WAVES) / GH;
   const size_t lds = (SPLIT ? 4 : 2) * (size_t)PROMPT_TILE_BYTES + (size_t)table_stride * sizeof(int);
-  auto kernel = attn_prompt_kernel<WAVES, SPLIT>;
+  auto kernel = attn_prompt_kernel<WAVES, SPLIT, CAP>;
   static size_t granted = 0;                     // per instantiation
   if (lds > granted) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -446,7 +457,8 @@ static int launch_prompt(const void* q, int q_stride, const void* k_cache, const
     if (page_size == (1 << b)) ps_shift = b;
   hipLaunchKernelGGL(kernel, grid, dim3(WAVES * QIL_WAVE), lds, s, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
                      (const bf16_t*)v_cache, block_tables, table_stride, cu_seqlens, seq_starts, (bf16_t*)out, heads,
-                     kv_heads, page_size, window, scale, GH, chunks, ps_shift, workspace, part_m, part_l, P, parts);
+                     kv_heads, page_size, window, scale, GH, chunks, ps_shift, workspace, part_m, part_l, P, parts,
+                     softcap);
   return (int)hipGetLastError();
 }
 
@@ -477,4 +489,20 @@ extern "C" int qil_attn_prompt(const void* q, int q_stride, const void* k_cache,
                                   total_rows, P, parts);
   return launch_prompt<4>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out, n_seqs,
                           max_query, heads, kv_heads, page_size, window, scale, s, (float*)workspace, total_rows, P, parts);
+}
+
+// The same with softly capped scores (blocks of 4 waves; keys in one part or in parts).
+extern "C" int qil_attn_prompt_capped(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                      const int* block_tables, int table_stride, const int* cu_seqlens,
+                                      const int* seq_starts, void* out, int n_seqs, int max_query, int heads, int kv_heads,
+                                      int page_size, int window, float scale, float softcap, void* workspace,
+                                      int total_rows, int P, int parts, hipStream_t s) {
+  if (n_seqs == 0 || max_query < 2) return 0;
+  if (!qil_attn_prompt_takes(PROMPT_D, page_size, table_stride) || heads % kv_heads || n_seqs > 65535 ||
+      (long)kv_heads * 2 * parts > 65535 || parts < 1 || !(softcap > 0.f) ||
+      (parts > 1 && (!workspace || total_rows < 1 || P < PROMPT_BK || P % PROMPT_BK)) || (parts == 1 && !out))
+    return -1;
+  return launch_prompt<4, false, true>(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts,
+                                       out, n_seqs, max_query, heads, kv_heads, page_size, window, scale, s,
+                                       (float*)workspace, total_rows, P, parts, softcap);
 }

@@ -522,6 +522,13 @@ extern "C" int qil_attn_tile_bf16(const void* q, int q_stride, const void* k_cac
                                   const int* seq_starts, void* out, int n_seqs, int max_query, int heads, int kv_heads,
                                   int d, int page_size, int window, float scale, hipStream_t s);
 
+extern "C" int qil_attn_prompt_takes(int d, int page_size, int table_stride);
+extern "C" int qil_attn_prompt_capped(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                                      const int* block_tables, int table_stride, const int* cu_seqlens,
+                                      const int* seq_starts, void* out, int n_seqs, int max_query, int heads, int kv_heads,
+                                      int page_size, int window, float scale, float softcap, void* workspace,
+                                      int total_rows, int P, int parts, hipStream_t s);
+
 // Keys in parts for this file's kernel (the float32 path, and bfloat16 sizes that the branch-free kernel does not
 // take): a portion of a prompt deep in a long context is a few row tiles, each with all its keys ahead of it one
 // after the other, on fewer blocks than the chip has CUs.  Returns the number of parts to cut the keys into (1: do
@@ -557,6 +564,11 @@ static int tile_dispatch(const void* q, int q_stride, const void* k_cache, const
                          int parts, float softcap) {
   if (n_seqs == 0 || max_query < 2) return 0;
   if (d % 8 || d < 8 || d > 256 || heads % kv_heads || n_seqs > 65535 || kv_heads * 2 > 65535) return -1;
+  // capped scores of bfloat16 heads of 128: the prompt kernel's capped form (keys in one part or in parts of whole tiles)
+  if (softcap > 0.f && dtype == QIL_BF16 && qil_attn_prompt_takes(d, page_size, table_stride) && (parts == 1 || P % 64 == 0))
+    return qil_attn_prompt_capped(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
+                                  n_seqs, max_query, heads, kv_heads, page_size, window, scale, softcap, workspace,
+                                  total_rows, P, parts, s);
   if (parts == 1 && softcap <= 0.f && dtype == QIL_BF16 && qil_attn_tile_bf16_takes(d, page_size, table_stride))
     return qil_attn_tile_bf16(q, q_stride, k_cache, v_cache, block_tables, table_stride, cu_seqlens, seq_starts, out,
                               n_seqs, max_query, heads, kv_heads, d, page_size, window, scale, s);

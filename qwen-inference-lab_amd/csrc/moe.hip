@@ -1,7 +1,7 @@
 // A routed feed-forward (mixture of experts): the router, the grouping of (token, chosen expert) pairs by expert, the
 // experts' two products on the matrix cores, and the weighted sum.
 //
-//   route    per token: logits z = W_r h in float32 (W_r float32, h as it comes), scores s = softmax(z) over all
+//   route    (two kernels: the logits, then the choice) per token: logits z = W_r h in float32 (W_r float32, h as it comes), scores s = softmax(z) over all
 //            outputs; choice scores c = s + correction; the outputs form `groups` equal groups of neighbours, a
 //            group's score is its largest c, and only the `keep` best groups stay (the others' c count as -inf);
 //            the `top` largest c are chosen (lowest index first among equals); the weights are their s, optionally
@@ -37,94 +37,120 @@ __device__ __forceinline__ void wave_argmax(float& v, int& at) {          // the
   }
 }
 
-template <typename T>
+// logits[n, e] = sum_i x[n, i] w[e, i] in float32.  grid (rows / 8, outputs / 4): a wave makes one output of eight rows, its
+// lanes along the width (a router row is read once for the eight); no LDS, no barrier.
+__device__ __forceinline__ float4 moe_load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 moe_load4(const bf16_t* p) {
+  const uint2 raw = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(raw.x << 16), __uint_as_float(raw.x & 0xffff0000u), __uint_as_float(raw.y << 16),
+                     __uint_as_float(raw.y & 0xffff0000u));
+}
+template <typename T, bool VEC>
 __global__ void __launch_bounds__(MOE_ROUTE_THREADS)
-moe_route_kernel(const T* __restrict__ x, int width, const float* __restrict__ w_router, const float* __restrict__ correction,
-                 int outputs, int groups, int keep, int top, int renormalize, int* __restrict__ chosen,
-                 float* __restrict__ weights) {
-  extern __shared__ float lds[];                        // [width] the row, [outputs] scores, [outputs] choice scores, [groups]
-  float* row = lds;
-  float* score = row + width;
+moe_logits_kernel(const T* __restrict__ x, int n, int width, const float* __restrict__ w_router, int outputs,
+                  float* __restrict__ logits) {
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  const int e = blockIdx.y * 4 + wave, row0 = blockIdx.x * 8;
+  if (e >= outputs) return;
+  const float* w = w_router + (size_t)e * width;
+  const T* rows[8];
+#pragma unroll
+  for (int r = 0; r < 8; ++r) rows[r] = x + (size_t)min(row0 + r, n - 1) * width;
+  float acc[8] = {};
+  if (VEC) {
+    for (int i = lane * 4; i < width; i += QIL_WAVE * 4) {
+      const float4 wv = moe_load4(w + i);
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const float4 xv = moe_load4(rows[r] + i);
+        acc[r] += xv.x * wv.x + xv.y * wv.y + xv.z * wv.z + xv.w * wv.w;
+      }
+    }
+  } else {
+    for (int i = lane; i < width; i += QIL_WAVE) {
+      const float wv = w[i];
+#pragma unroll
+      for (int r = 0; r < 8; ++r) acc[r] += ld(rows[r] + i) * wv;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    const float total = wave_sum(acc[r]);
+    if (lane == 0 && row0 + r < n) logits[(size_t)(row0 + r) * outputs + e] = total;
+  }
+}
+
+// The choice from the logits: a wave a row, four rows a block (every wave walks the same steps, so the barriers
+// between a wave's writes to its part of LDS and its reads are met by all).
+__global__ void __launch_bounds__(MOE_ROUTE_THREADS)
+moe_select_kernel(const float* __restrict__ logits, int n, const float* __restrict__ correction, int outputs, int groups,
+                  int keep, int top, int renormalize, int* __restrict__ chosen, float* __restrict__ weights) {
+  extern __shared__ float lds[];                        // per wave: [outputs] scores, [outputs] choice scores, [groups]
+  const int lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
+  float* score = lds + (size_t)wave * (2 * outputs + groups);
   float* choice = score + outputs;
   float* group_best = choice + outputs;
-  const int n = blockIdx.x, lane = threadIdx.x & (QIL_WAVE - 1), wave = threadIdx.x / QIL_WAVE;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) row[i] = ld(x + (size_t)n * width + i);
-  __syncthreads();
-  for (int e = wave; e < outputs; e += MOE_ROUTE_THREADS / QIL_WAVE) {
-    const float* w = w_router + (size_t)e * width;
-    float dot = 0.f;
-    for (int i = lane; i < width; i += QIL_WAVE) dot += row[i] * w[i];
-    dot = wave_sum(dot);
-    if (lane == 0) score[e] = dot;
-  }
-  __syncthreads();
-  // the rest is one wave's work; the others keep it company at the barriers between its steps
-  const bool mine = wave == 0;
-  if (mine) {
-    float top_logit = -INFINITY;
-    for (int e = lane; e < outputs; e += QIL_WAVE) top_logit = fmaxf(top_logit, score[e]);
-    top_logit = wave_max(top_logit);
-    float total = 0.f;
-    for (int e = lane; e < outputs; e += QIL_WAVE) total += expf(score[e] - top_logit);
-    total = wave_sum(total);
-    for (int e = lane; e < outputs; e += QIL_WAVE) {      // (a lane meets its own elements again)
-      const float s = expf(score[e] - top_logit) / total;
-      score[e] = s;
-      choice[e] = s + (correction ? correction[e] : 0.f);
-    }
+  const int n_row = blockIdx.x * (MOE_ROUTE_THREADS / QIL_WAVE) + wave;
+  const bool live = n_row < n;
+  const float* z = logits + (size_t)min(n_row, n - 1) * outputs;
+  float top_logit = -INFINITY;
+  for (int e = lane; e < outputs; e += QIL_WAVE) top_logit = fmaxf(top_logit, z[e]);
+  top_logit = wave_max(top_logit);
+  float total = 0.f;
+  for (int e = lane; e < outputs; e += QIL_WAVE) total += expf(z[e] - top_logit);
+  total = wave_sum(total);
+  for (int e = lane; e < outputs; e += QIL_WAVE) {
+    const float s = expf(z[e] - top_logit) / total;
+    score[e] = s;
+    choice[e] = s + (correction ? correction[e] : 0.f);
   }
   __syncthreads();
   if (groups > 1 && keep < groups) {
     const int size = outputs / groups;
-    if (mine)
-      for (int g = lane; g < groups; g += QIL_WAVE) {
-        float best = -INFINITY;
-        for (int e = g * size; e < (g + 1) * size; ++e) best = fmaxf(best, choice[e]);
-        group_best[g] = best;
-      }
+    for (int g = lane; g < groups; g += QIL_WAVE) {
+      float best = -INFINITY;
+      for (int e = g * size; e < (g + 1) * size; ++e) best = fmaxf(best, choice[e]);
+      group_best[g] = best;
+    }
     __syncthreads();
     // the `keep` best groups are marked by +inf in their place, one after the other
     for (int round = 0; round < keep; ++round) {
       float v = -INFINITY;
       int at = 0x7fffffff;
-      if (mine) {
-        for (int g = lane; g < groups; g += QIL_WAVE) {
-          const float gv = group_best[g];
-          if (gv != INFINITY && (gv > v || at == 0x7fffffff)) { v = gv; at = g; }
-        }
-        wave_argmax(v, at);
+      for (int g = lane; g < groups; g += QIL_WAVE) {
+        const float gv = group_best[g];
+        if (gv != INFINITY && (gv > v || at == 0x7fffffff)) { v = gv; at = g; }
       }
+      wave_argmax(v, at);
       __syncthreads();
-      if (mine && lane == 0 && at != 0x7fffffff) group_best[at] = INFINITY;
+      if (lane == 0 && at != 0x7fffffff) group_best[at] = INFINITY;
       __syncthreads();
     }
-    if (mine)
-      for (int e = lane; e < outputs; e += QIL_WAVE)
-        if (group_best[e / size] != INFINITY) choice[e] = -INFINITY;
+    for (int e = lane; e < outputs; e += QIL_WAVE)
+      if (group_best[e / size] != INFINITY) choice[e] = -INFINITY;
     __syncthreads();
   }
-  float sum = 0.f;
+  float sum = 0.f, mine = 0.f;
   for (int round = 0; round < top; ++round) {
     float v = -INFINITY;
     int at = 0x7fffffff;
-    if (mine) {
-      for (int e = lane; e < outputs; e += QIL_WAVE) {
-        const float c = choice[e];
-        if (c == c && c != INFINITY && (c > v || at == 0x7fffffff)) { v = c; at = e; }   // +inf marks what is taken
-      }
-      wave_argmax(v, at);
-      if (at == 0x7fffffff) at = 0;
-      sum += score[at];
+    for (int e = lane; e < outputs; e += QIL_WAVE) {
+      const float c = choice[e];
+      if (c == c && c != INFINITY && (c > v || at == 0x7fffffff)) { v = c; at = e; }   // +inf marks what is taken
     }
+    wave_argmax(v, at);
+    if (at == 0x7fffffff) at = 0;
+    const float s = score[at];
+    sum += s;
+    if (lane == round) mine = s;
     __syncthreads();
-    if (mine && lane == 0) {
-      chosen[(size_t)n * top + round] = at;
-      weights[(size_t)n * top + round] = score[at];
+    if (lane == 0) {
+      if (live) chosen[(size_t)n_row * top + round] = at;
       choice[at] = INFINITY;
     }
     __syncthreads();
   }
-  if (renormalize && mine && lane < top) weights[(size_t)n * top + lane] = score[chosen[(size_t)n * top + lane]] / sum;
+  if (live && lane < top) weights[(size_t)n_row * top + lane] = renormalize ? mine / sum : mine;
 }
 
 // ------------------------------------------------------------------------------------------------ align
@@ -233,17 +259,26 @@ moe_gate_up_kernel(const T* __restrict__ x, int width, const T* __restrict__ w, 
   moe_f32x4 acc_g[MT], acc_u[MT];
 #pragma unroll
   for (int m = 0; m < MT; ++m) acc_g[m] = acc_u[m] = (moe_f32x4){0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < width; k0 += KC) {
-    const int k = k0 + kq * EPL;
-    const typename Frag<T>::raw bg = load_frag<T, ALIGNED>(g_row, k, width), bu = load_frag<T, ALIGNED>(u_row, k, width);
-    typename Frag<T>::raw a[MT];
+  // the fragments of the next step are on their way while this step's products run
+  typename Frag<T>::raw bg = load_frag<T, ALIGNED>(g_row, kq * EPL, width), bu = load_frag<T, ALIGNED>(u_row, kq * EPL, width);
+  typename Frag<T>::raw a[MT];
 #pragma unroll
-    for (int m = 0; m < MT; ++m) a[m] = load_frag<T, ALIGNED>(a_row[m], k, width);
+  for (int m = 0; m < MT; ++m) a[m] = load_frag<T, ALIGNED>(a_row[m], kq * EPL, width);
+  for (int k0 = 0; k0 < width; k0 += KC) {
+    const int k = k0 + KC + kq * EPL;                    // (past the end: zeros, never used)
+    const typename Frag<T>::raw bg_next = load_frag<T, ALIGNED>(g_row, k, width), bu_next = load_frag<T, ALIGNED>(u_row, k, width);
+    typename Frag<T>::raw a_next[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) a_next[m] = load_frag<T, ALIGNED>(a_row[m], k, width);
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       Frag<T>::mma(acc_g[m], a[m], bg);
       Frag<T>::mma(acc_u[m], a[m], bu);
     }
+    bg = bg_next;
+    bu = bu_next;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) a[m] = a_next[m];
   }
   if (col0 + r >= ff) return;
 #pragma unroll
@@ -278,17 +313,25 @@ moe_down_kernel(const T* __restrict__ hidden, int ff, const T* __restrict__ w, i
   moe_f32x4 acc[MT][2];
 #pragma unroll
   for (int m = 0; m < MT; ++m) acc[m][0] = acc[m][1] = (moe_f32x4){0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < ff; k0 += KC) {
-    const int k = k0 + kq * EPL;
-    const typename Frag<T>::raw b0 = load_frag<T, ALIGNED>(b_row[0], k, ff), b1 = load_frag<T, ALIGNED>(b_row[1], k, ff);
-    typename Frag<T>::raw a[MT];
+  typename Frag<T>::raw b0 = load_frag<T, ALIGNED>(b_row[0], kq * EPL, ff), b1 = load_frag<T, ALIGNED>(b_row[1], kq * EPL, ff);
+  typename Frag<T>::raw a[MT];
 #pragma unroll
-    for (int m = 0; m < MT; ++m) a[m] = load_frag<T, ALIGNED>(a_row[m], k, ff);
+  for (int m = 0; m < MT; ++m) a[m] = load_frag<T, ALIGNED>(a_row[m], kq * EPL, ff);
+  for (int k0 = 0; k0 < ff; k0 += KC) {
+    const int k = k0 + KC + kq * EPL;
+    const typename Frag<T>::raw b0_next = load_frag<T, ALIGNED>(b_row[0], k, ff), b1_next = load_frag<T, ALIGNED>(b_row[1], k, ff);
+    typename Frag<T>::raw a_next[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) a_next[m] = load_frag<T, ALIGNED>(a_row[m], k, ff);
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       Frag<T>::mma(acc[m][0], a[m], b0);
       Frag<T>::mma(acc[m][1], a[m], b1);
     }
+    b0 = b0_next;
+    b1 = b1_next;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) a[m] = a_next[m];
   }
 #pragma unroll
   for (int m = 0; m < MT; ++m)
@@ -300,6 +343,115 @@ moe_down_kernel(const T* __restrict__ hidden, int ff, const T* __restrict__ w, i
 #pragma unroll
       for (int t = 0; t < 2; ++t)
         if (col0 + t * 16 + r < width) out[col0 + t * 16 + r] = acc[m][t][i];
+    }
+}
+
+// The two products for steps with many pairs an expert (bfloat16, tiles of 64 pairs, rows of whole 16-byte pieces): a
+// block makes 64 pairs by 256 result columns, a wave 64 by 64 (16 tiles of 16 x 16, v_mfma_f32_16x16x32_bf16).  A stage
+// is 64 columns of K: every thread fetches its 16-byte pieces of the stage's A rows (64 x 128 bytes) and B rows (256 x
+// 128 bytes: whole cache lines) into registers while the stage before is multiplied, then the block puts them into LDS
+// (rows 144 bytes apart, so that the 16 rows of a fragment read fall on all banks) and the waves read their fragments
+// from there: a weight is read from memory once a block, a pair's row once a block.
+// GATED: A rows are the pairs' rows of x, the result columns are 128 gate columns and the same 128 up columns of the
+// expert (a wave owns 32 of each), and the block writes act(gate, up) for 128 hidden columns.  Otherwise A rows are the
+// places' rows of hidden, the result columns are 256 of the expert's down matrix, written to the pairs' rows of y.
+#define MOE_TILE_ROW 144                                  // bytes of a staged row: 128 and 16 to spread the banks
+#define MOE_TILE_LDS ((64 + 256) * MOE_TILE_ROW)
+template <bool GATED>
+__global__ void __launch_bounds__(256)
+moe_tile_kernel(const bf16_t* __restrict__ a_base, const bf16_t* __restrict__ w, int K, int columns,
+                const int* __restrict__ tiles, int max_tiles, const int* __restrict__ places, int top,
+                bf16_t* __restrict__ hidden, float* __restrict__ y, int act, float limit, float alpha) {
+  extern __shared__ __align__(16) unsigned char tile_lds[];
+  unsigned char* a_lds = tile_lds;
+  unsigned char* b_lds = tile_lds + 64 * MOE_TILE_ROW;
+  const int tile = blockIdx.x, rows = tiles[2 * max_tiles + tile];
+  if (rows == 0) return;
+  const int e = tiles[tile], begin = tiles[max_tiles + tile];
+  const int tid = threadIdx.x, lane = tid & (QIL_WAVE - 1), wave = tid / QIL_WAVE;
+  const int r = lane & 15, kq = lane >> 4;
+  const int c0 = blockIdx.y * (GATED ? 128 : 256);        // first hidden column, or first output column
+  // what this thread fetches of a stage: piece tid % 8 of the rows tid / 8 + 32 j
+  const int piece = tid & 7, row0 = tid >> 3;
+  const bf16_t* a_src[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int local = min(row0 + 32 * j, rows - 1);
+    a_src[j] = GATED ? a_base + (size_t)(places[begin + local] / top) * K : a_base + (size_t)(begin + local) * K;
+  }
+  const bf16_t* b_src[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int rb = row0 + 32 * j;
+    if (GATED) b_src[j] = w + ((size_t)(e * 2 + (rb >> 7)) * columns + min(c0 + (rb & 127), columns - 1)) * K;
+    else b_src[j] = w + ((size_t)e * columns + min(c0 + rb, columns - 1)) * K;
+  }
+  qil_u32x4 fetched_a[2], fetched_b[8];
+  auto fetch = [&](int k0) {
+    const int k = k0 + piece * 8;
+    const bool inside = k < K;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      fetched_a[j] = inside ? *reinterpret_cast<const qil_u32x4*>(a_src[j] + k) : (qil_u32x4){0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      fetched_b[j] = inside ? *reinterpret_cast<const qil_u32x4*>(b_src[j] + k) : (qil_u32x4){0u, 0u, 0u, 0u};
+  };
+  // the rows of B whose tiles this wave multiplies: GATED 32 gate rows and the 32 up rows of the same columns
+  int b_tile[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) b_tile[t] = GATED ? (t >> 1) * 128 + wave * 32 + (t & 1) * 16 : wave * 64 + t * 16;
+  moe_f32x4 acc[4][4];
+#pragma unroll
+  for (int m = 0; m < 4; ++m)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[m][t] = (moe_f32x4){0.f, 0.f, 0.f, 0.f};
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += 64) {
+    __syncthreads();                                      // the stage before has been read
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      *reinterpret_cast<qil_u32x4*>(a_lds + (row0 + 32 * j) * MOE_TILE_ROW + piece * 16) = fetched_a[j];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      *reinterpret_cast<qil_u32x4*>(b_lds + (row0 + 32 * j) * MOE_TILE_ROW + piece * 16) = fetched_b[j];
+    __syncthreads();
+    if (k0 + 64 < K) fetch(k0 + 64);                      // on its way while this stage is multiplied
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      qil_u32x4 a[4], b[4];
+#pragma unroll
+      for (int m = 0; m < 4; ++m)
+        a[m] = *reinterpret_cast<const qil_u32x4*>(a_lds + (m * 16 + r) * MOE_TILE_ROW + ks * 64 + kq * 16);
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        b[t] = *reinterpret_cast<const qil_u32x4*>(b_lds + (b_tile[t] + r) * MOE_TILE_ROW + ks * 64 + kq * 16);
+#pragma unroll
+      for (int m = 0; m < 4; ++m)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) Frag<bf16_t>::mma(acc[m][t], a[m], b[t]);
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < 4; ++m)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int local = m * 16 + 4 * kq + i;
+      if (local >= rows) continue;
+      if (GATED) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const int col = c0 + wave * 32 + t * 16 + r;
+          if (col < columns) st(hidden + (size_t)(begin + local) * columns + col, gated_act(acc[m][t][i], acc[m][2 + t][i], act, limit, alpha));
+        }
+      } else {
+        float* out = y + (size_t)places[begin + local] * columns;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int col = c0 + wave * 64 + t * 16 + r;
+          if (col < columns) out[col] = acc[m][t][i];
+        }
+      }
     }
 }
 
@@ -325,22 +477,28 @@ extern "C" {
 int qil_moe_takes(int width, int outputs, int experts, int groups, int keep, int top) {
   return width >= 1 && outputs >= 1 && outputs <= MOE_MAX_OUTPUTS && experts >= 0 && experts <= outputs && groups >= 1 &&
          outputs % groups == 0 && keep >= 1 && keep <= groups && top >= 1 && top <= outputs && top <= QIL_WAVE &&
-         (size_t)(width + 2 * outputs + groups) * sizeof(float) <= 64 * 1024;
+         (size_t)(MOE_ROUTE_THREADS / QIL_WAVE) * (2 * outputs + groups) * sizeof(float) <= 64 * 1024;
 }
 
 // x [n, width] (dtype), w_router float32 [outputs, width], correction float32 [outputs] or null -> chosen int32
-// [n, top], weights float32 [n, top].
-int qil_moe_route(const void* x, int dtype, const float* w_router, const float* correction, int* chosen, float* weights,
-                  int n, int width, int outputs, int groups, int keep, int top, int renormalize, hipStream_t s) {
+// [n, top], weights float32 [n, top].  logits: float32 scratch [n, outputs].
+int qil_moe_route(const void* x, int dtype, const float* w_router, const float* correction, float* logits, int* chosen,
+                  float* weights, int n, int width, int outputs, int groups, int keep, int top, int renormalize,
+                  hipStream_t s) {
   if (n == 0) return 0;
-  if (!qil_moe_takes(width, outputs, 0, groups, keep, top)) return -1;
-  const size_t lds = (size_t)(width + 2 * outputs + groups) * sizeof(float);
-  if (dtype == QIL_F32)
-    hipLaunchKernelGGL(moe_route_kernel<float>, dim3(n), dim3(MOE_ROUTE_THREADS), lds, s, (const float*)x, width, w_router,
-                       correction, outputs, groups, keep, top, renormalize, chosen, weights);
-  else
-    hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(n), dim3(MOE_ROUTE_THREADS), lds, s, (const bf16_t*)x, width,
-                       w_router, correction, outputs, groups, keep, top, renormalize, chosen, weights);
+  if (!qil_moe_takes(width, outputs, 0, groups, keep, top) || !logits) return -1;
+  const dim3 g_logits((n + 7) / 8, (outputs + 3) / 4);
+  const bool vec = width % 4 == 0 && (((uintptr_t)x | (uintptr_t)w_router) % 16) == 0;
+#define QIL_LOGITS(T, VEC)                                                                                            \
+  hipLaunchKernelGGL((moe_logits_kernel<T, VEC>), g_logits, dim3(MOE_ROUTE_THREADS), 0, s, (const T*)x, n, width,      \
+                     w_router, outputs, logits)
+  if (dtype == QIL_F32) { if (vec) QIL_LOGITS(float, true); else QIL_LOGITS(float, false); }
+  else { if (vec) QIL_LOGITS(bf16_t, true); else QIL_LOGITS(bf16_t, false); }
+#undef QIL_LOGITS
+  const int per_block = MOE_ROUTE_THREADS / QIL_WAVE;
+  const size_t lds = (size_t)per_block * (2 * outputs + groups) * sizeof(float);
+  hipLaunchKernelGGL(moe_select_kernel, dim3((n + per_block - 1) / per_block), dim3(MOE_ROUTE_THREADS), lds, s, logits, n,
+                     correction, outputs, groups, keep, top, renormalize, chosen, weights);
   QIL_RETURN_LAUNCH_STATUS();
 }
 
@@ -368,6 +526,21 @@ int qil_moe_experts(const void* x, int dtype, const int* chosen, const float* we
     const bool aligned = width % epl == 0 && ff % epl == 0 &&
                          (((uintptr_t)x | (uintptr_t)w_gate_up | (uintptr_t)w_down | (uintptr_t)hidden) % 16) == 0;
     const dim3 g_up(max_tiles, (ff + 63) / 64), g_down(max_tiles, (width + 127) / 128);
+    if (dtype == QIL_BF16 && tile_rows == 64 && aligned && width % 8 == 0 && ff % 8 == 0) {
+      static bool granted = false;                        // (both instantiations, once)
+      if (!granted) {
+        hipError_t a = hipFuncSetAttribute((const void*)moe_tile_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, MOE_TILE_LDS);
+        hipError_t b = hipFuncSetAttribute((const void*)moe_tile_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, MOE_TILE_LDS);
+        if (a != hipSuccess || b != hipSuccess) return (int)(a != hipSuccess ? a : b);
+        granted = true;
+      }
+      hipLaunchKernelGGL(moe_tile_kernel<true>, dim3(max_tiles, (ff + 127) / 128), dim3(256), MOE_TILE_LDS, s,
+                         (const bf16_t*)x, (const bf16_t*)w_gate_up, width, ff, tiles, max_tiles, places, top,
+                         (bf16_t*)hidden, (float*)nullptr, act, limit, alpha);
+      hipLaunchKernelGGL(moe_tile_kernel<false>, dim3(max_tiles, (width + 255) / 256), dim3(256), MOE_TILE_LDS, s,
+                         (const bf16_t*)hidden, (const bf16_t*)w_down, ff, width, tiles, max_tiles, places, top,
+                         (bf16_t*)nullptr, y, act, limit, alpha);
+    } else {
 #define QIL_MOE(T, MT, ALIGNED)                                                                                       \
   do {                                                                                                                \
     hipLaunchKernelGGL((moe_gate_up_kernel<T, MT, ALIGNED>), g_up, dim3(256), 0, s, (const T*)x, width,                \
@@ -383,6 +556,7 @@ int qil_moe_experts(const void* x, int dtype, const int* chosen, const float* we
     if (dtype == QIL_F32) QIL_MOE_T(float); else QIL_MOE_T(bf16_t);
 #undef QIL_MOE_T
 #undef QIL_MOE
+    }
   }
   const int threads = width >= 1024 ? 256 : 64;
   if (dtype == QIL_F32)

@@ -1112,8 +1112,10 @@ def moe_route(x, router, correction, *, groups, keep, top, renormalize=False):
         raise UnsupportedShape(f'moe_route: {outputs} outputs in {groups} groups ({keep} kept), top {top}, width {width}')
     chosen = torch.empty((n, top), dtype=torch.int32, device=x.device)
     weights = torch.empty((n, top), dtype=torch.float32, device=x.device)
-    _check(lib.qil_moe_route(_ptr(x), _code(x.dtype), _ptr(router), _ptr(correction), _ptr(chosen), _ptr(weights), n, width,
-                             outputs, groups, keep, top, int(bool(renormalize)), _stream()), 'moe_route')
+    logits = torch.empty((n, outputs), dtype=torch.float32, device=x.device)
+    _check(lib.qil_moe_route(_ptr(x), _code(x.dtype), _ptr(router), _ptr(correction), _ptr(logits), _ptr(chosen),
+                             _ptr(weights), n, width, outputs, groups, keep, top, int(bool(renormalize)), _stream()),
+           'moe_route')
     return chosen, weights
 
 

@@ -321,7 +321,7 @@ def _declare(lib):
     lib.qil_post_norm_add_norm.restype = i
     lib.qil_moe_takes.argtypes = [i, i, i, i, i, i]
     lib.qil_moe_takes.restype = i
-    lib.qil_moe_route.argtypes = [p, i, p, p, p, p, i, i, i, i, i, i, i, p]
+    lib.qil_moe_route.argtypes = [p, i, p, p, p, p, p, i, i, i, i, i, i, i, p]
     lib.qil_moe_route.restype = i
     lib.qil_moe_tile_rows.argtypes = [i, i]
     lib.qil_moe_tile_rows.restype = i

@@ -253,6 +253,7 @@ def test_the_router_by_hand():
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('sizes', [dict(n=5, width=40, ff=16, experts=6, identity=2, top=3),
                                    dict(n=300, width=64, ff=48, experts=3, identity=0, top=2),       # tiles of 64 pairs
+                                   dict(n=260, width=200, ff=144, experts=2, identity=1, top=2),    # stages of 64 columns with a rest
                                    dict(n=70, width=36, ff=32, experts=4, identity=4, top=4),        # width no multiple of 8
                                    dict(n=1, width=256, ff=64, experts=12, identity=2, top=3),
                                    dict(n=33, width=136, ff=80, experts=1, identity=1, top=2)])
