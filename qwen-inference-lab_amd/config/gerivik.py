@@ -5,7 +5,7 @@
     embedding      {'scale'}: what an embedded token is multiplied by
     layers         list; each entry: 'type' (the mixer: 'attention' | 'gla'), 'mixer' (its sizes and constants), 'mlp'
                    (null, or {'kind': 'moe', 'expert': {'ff', 'limit'}, 'router': {'experts', 'identity', 'top',
-                   'groups': {'count', 'keep'}}}) and optionally 'weights_of': j, the index of an earlier layer with
+                   'groups': {'count', 'keep'}}}) and optionally 'weights_of': j, the index of another layer with
                    tensors of its own whose tensors this layer uses (with a cache or state of its own); the rest of
                    such an entry equals layer j's
     norm           {'eps'}
@@ -76,8 +76,9 @@ def _check_layer(index, layer, layers):
                               f'{keep} can hold {router["top"]} choices')
     if 'weights_of' in layer:
         source = layer['weights_of']
-        if type(source) is not int or not 0 <= source < index or 'weights_of' in layers[source]:
-            raise ConfigError(f'{where}.weights_of must name an earlier layer that has tensors of its own')
+        if type(source) is not int or not 0 <= source < len(layers) or source == index or \
+                not isinstance(layers[source], dict) or 'weights_of' in layers[source]:
+            raise ConfigError(f'{where}.weights_of must name another layer that has tensors of its own')
         if {k: v for k, v in layer.items() if k != 'weights_of'} != layers[source]:
             raise ConfigError(f'{where}: a layer that uses the tensors of layer {source} must equal it otherwise')
 

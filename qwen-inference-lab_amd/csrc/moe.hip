@@ -347,9 +347,10 @@ moe_down_kernel(const T* __restrict__ hidden, int ff, const T* __restrict__ w, i
 }
 
 // The two products for steps with many pairs an expert (bfloat16, tiles of 64 pairs, rows of whole 16-byte pieces): a
-// block makes 64 pairs by 256 result columns, a wave 64 by 64 (16 tiles of 16 x 16, v_mfma_f32_16x16x32_bf16).  A stage
-// is 64 columns of K: every thread fetches its 16-byte pieces of the stage's A rows (64 x 128 bytes) and B rows (256 x
-// 128 bytes: whole cache lines) into registers while the stage before is multiplied, then the block puts them into LDS
+// block of eight waves makes 64 pairs by 256 result columns, a wave 32 by 64 (8 tiles of 16 x 16,
+// v_mfma_f32_16x16x32_bf16).  A stage is 64 columns of K: every thread fetches its 16-byte pieces of the stage's A rows
+// (64 x 128 bytes) and B rows (256 x 128 bytes: whole cache lines) into registers while the two stages before are
+// multiplied, then the block puts them into LDS
 // (rows 144 bytes apart, so that the 16 rows of a fragment read fall on all banks) and the waves read their fragments
 // from there: a weight is read from memory once a block, a pair's row once a block.
 // GATED: A rows are the pairs' rows of x, the result columns are 128 gate columns and the same 128 up columns of the
@@ -357,98 +358,115 @@ moe_down_kernel(const T* __restrict__ hidden, int ff, const T* __restrict__ w, i
 // places' rows of hidden, the result columns are 256 of the expert's down matrix, written to the pairs' rows of y.
 #define MOE_TILE_ROW 144                                  // bytes of a staged row: 128 and 16 to spread the banks
 #define MOE_TILE_LDS ((64 + 256) * MOE_TILE_ROW)
+#define MOE_TILE_THREADS 512
+struct MoeFetched { qil_u32x4 a, b[4]; };                 // a thread's pieces of one stage: one of A, four of B
 template <bool GATED>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(MOE_TILE_THREADS, 2)
 moe_tile_kernel(const bf16_t* __restrict__ a_base, const bf16_t* __restrict__ w, int K, int columns,
                 const int* __restrict__ tiles, int max_tiles, const int* __restrict__ places, int top,
-                bf16_t* __restrict__ hidden, float* __restrict__ y, int act, float limit, float alpha) {
+                bf16_t* __restrict__ hidden, float* __restrict__ y, int act, float limit, float alpha, int column_blocks) {
   extern __shared__ __align__(16) unsigned char tile_lds[];
   unsigned char* a_lds = tile_lds;
   unsigned char* b_lds = tile_lds + 64 * MOE_TILE_ROW;
-  const int tile = blockIdx.x, rows = tiles[2 * max_tiles + tile];
+  // Blocks go to the chip's 8 XCDs in turn, and every XCD has an L2 of its own: the block numbers are turned so that
+  // an XCD works through a run of (column block, tile) pairs with the tile moving fastest.  The tiles of one expert
+  // follow each other, so its weights come from memory once an XCD and from that XCD's L2 for the expert's other tiles
+  // (numbered in launch order, every XCD fetched every expert's weights: 2.2 GB through the fabric for 0.6 GB of weights).
+  const int per_xcd = gridDim.x / 8;
+  const int turned = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (turned >= max_tiles * column_blocks) return;
+  const int tile = turned % max_tiles, column_block = turned / max_tiles;
+  const int rows = tiles[2 * max_tiles + tile];
   if (rows == 0) return;
   const int e = tiles[tile], begin = tiles[max_tiles + tile];
   const int tid = threadIdx.x, lane = tid & (QIL_WAVE - 1), wave = tid / QIL_WAVE;
   const int r = lane & 15, kq = lane >> 4;
-  const int c0 = blockIdx.y * (GATED ? 128 : 256);        // first hidden column, or first output column
-  // what this thread fetches of a stage: piece tid % 8 of the rows tid / 8 + 32 j
+  const int half = wave >> 2, quarter = wave & 3;         // the wave's 32 of the 64 pairs, its 64 of the 256 columns
+  const int c0 = column_block * (GATED ? 128 : 256);      // first hidden column, or first output column
+  // what this thread fetches of a stage: piece tid % 8 of row tid / 8 of A and of the rows tid / 8 + 64 j of B
   const int piece = tid & 7, row0 = tid >> 3;
-  const bf16_t* a_src[2];
+  const int local0 = min(row0, rows - 1);
+  const bf16_t* a_src = GATED ? a_base + (size_t)(places[begin + local0] / top) * K : a_base + (size_t)(begin + local0) * K;
+  const bf16_t* b_src[4];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int local = min(row0 + 32 * j, rows - 1);
-    a_src[j] = GATED ? a_base + (size_t)(places[begin + local] / top) * K : a_base + (size_t)(begin + local) * K;
-  }
-  const bf16_t* b_src[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int rb = row0 + 32 * j;
+  for (int j = 0; j < 4; ++j) {
+    const int rb = row0 + 64 * j;
     if (GATED) b_src[j] = w + ((size_t)(e * 2 + (rb >> 7)) * columns + min(c0 + (rb & 127), columns - 1)) * K;
     else b_src[j] = w + ((size_t)e * columns + min(c0 + rb, columns - 1)) * K;
   }
-  qil_u32x4 fetched_a[2], fetched_b[8];
-  auto fetch = [&](int k0) {
+  auto fetch = [&](MoeFetched& f, int k0) {
     const int k = k0 + piece * 8;
     const bool inside = k < K;
+    f.a = inside ? *reinterpret_cast<const qil_u32x4*>(a_src + k) : (qil_u32x4){0u, 0u, 0u, 0u};
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
-      fetched_a[j] = inside ? *reinterpret_cast<const qil_u32x4*>(a_src[j] + k) : (qil_u32x4){0u, 0u, 0u, 0u};
+    for (int j = 0; j < 4; ++j)
+      f.b[j] = inside ? *reinterpret_cast<const qil_u32x4*>(b_src[j] + k) : (qil_u32x4){0u, 0u, 0u, 0u};
+  };
+  auto put = [&](const MoeFetched& f) {
+    *reinterpret_cast<qil_u32x4*>(a_lds + row0 * MOE_TILE_ROW + piece * 16) = f.a;
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      fetched_b[j] = inside ? *reinterpret_cast<const qil_u32x4*>(b_src[j] + k) : (qil_u32x4){0u, 0u, 0u, 0u};
+    for (int j = 0; j < 4; ++j) *reinterpret_cast<qil_u32x4*>(b_lds + (row0 + 64 * j) * MOE_TILE_ROW + piece * 16) = f.b[j];
   };
   // the rows of B whose tiles this wave multiplies: GATED 32 gate rows and the 32 up rows of the same columns
   int b_tile[4];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) b_tile[t] = GATED ? (t >> 1) * 128 + wave * 32 + (t & 1) * 16 : wave * 64 + t * 16;
-  moe_f32x4 acc[4][4];
+  for (int t = 0; t < 4; ++t) b_tile[t] = GATED ? (t >> 1) * 128 + quarter * 32 + (t & 1) * 16 : quarter * 64 + t * 16;
+  moe_f32x4 acc[2][4];
 #pragma unroll
-  for (int m = 0; m < 4; ++m)
+  for (int m = 0; m < 2; ++m)
 #pragma unroll
     for (int t = 0; t < 4; ++t) acc[m][t] = (moe_f32x4){0.f, 0.f, 0.f, 0.f};
-  fetch(0);
-  for (int k0 = 0; k0 < K; k0 += 64) {
-    __syncthreads();                                      // the stage before has been read
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-      *reinterpret_cast<qil_u32x4*>(a_lds + (row0 + 32 * j) * MOE_TILE_ROW + piece * 16) = fetched_a[j];
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-      *reinterpret_cast<qil_u32x4*>(b_lds + (row0 + 32 * j) * MOE_TILE_ROW + piece * 16) = fetched_b[j];
-    __syncthreads();
-    if (k0 + 64 < K) fetch(k0 + 64);                      // on its way while this stage is multiplied
+  auto multiply = [&]() {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      qil_u32x4 a[4], b[4];
+      qil_u32x4 a[2], b[4];
 #pragma unroll
-      for (int m = 0; m < 4; ++m)
-        a[m] = *reinterpret_cast<const qil_u32x4*>(a_lds + (m * 16 + r) * MOE_TILE_ROW + ks * 64 + kq * 16);
+      for (int m = 0; m < 2; ++m)
+        a[m] = *reinterpret_cast<const qil_u32x4*>(a_lds + (half * 32 + m * 16 + r) * MOE_TILE_ROW + ks * 64 + kq * 16);
 #pragma unroll
       for (int t = 0; t < 4; ++t)
         b[t] = *reinterpret_cast<const qil_u32x4*>(b_lds + (b_tile[t] + r) * MOE_TILE_ROW + ks * 64 + kq * 16);
 #pragma unroll
-      for (int m = 0; m < 4; ++m)
+      for (int m = 0; m < 2; ++m)
 #pragma unroll
         for (int t = 0; t < 4; ++t) Frag<bf16_t>::mma(acc[m][t], a[m], b[t]);
     }
+  };
+  // two stages are on their way while a stage is multiplied (a trip to memory takes longer than one stage's products)
+  MoeFetched even, odd;
+  fetch(even, 0);
+  fetch(odd, 64);
+  for (int k0 = 0; k0 < K; k0 += 128) {
+    __syncthreads();                                      // the stage before has been read
+    put(even);
+    __syncthreads();
+    fetch(even, k0 + 128);                                // (past the end: zeros, no access)
+    multiply();
+    if (k0 + 64 < K) {
+      __syncthreads();
+      put(odd);
+      __syncthreads();
+      fetch(odd, k0 + 192);
+      multiply();
+    }
   }
 #pragma unroll
-  for (int m = 0; m < 4; ++m)
+  for (int m = 0; m < 2; ++m)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int local = m * 16 + 4 * kq + i;
+      const int local = half * 32 + m * 16 + 4 * kq + i;
       if (local >= rows) continue;
       if (GATED) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-          const int col = c0 + wave * 32 + t * 16 + r;
+          const int col = c0 + quarter * 32 + t * 16 + r;
           if (col < columns) st(hidden + (size_t)(begin + local) * columns + col, gated_act(acc[m][t][i], acc[m][2 + t][i], act, limit, alpha));
         }
       } else {
         float* out = y + (size_t)places[begin + local] * columns;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          const int col = c0 + wave * 64 + t * 16 + r;
+          const int col = c0 + quarter * 64 + t * 16 + r;
           if (col < columns) out[col] = acc[m][t][i];
         }
       }
@@ -534,12 +552,13 @@ int qil_moe_experts(const void* x, int dtype, const int* chosen, const float* we
         if (a != hipSuccess || b != hipSuccess) return (int)(a != hipSuccess ? a : b);
         granted = true;
       }
-      hipLaunchKernelGGL(moe_tile_kernel<true>, dim3(max_tiles, (ff + 127) / 128), dim3(256), MOE_TILE_LDS, s,
-                         (const bf16_t*)x, (const bf16_t*)w_gate_up, width, ff, tiles, max_tiles, places, top,
-                         (bf16_t*)hidden, (float*)nullptr, act, limit, alpha);
-      hipLaunchKernelGGL(moe_tile_kernel<false>, dim3(max_tiles, (width + 255) / 256), dim3(256), MOE_TILE_LDS, s,
-                         (const bf16_t*)hidden, (const bf16_t*)w_down, ff, width, tiles, max_tiles, places, top,
-                         (bf16_t*)nullptr, y, act, limit, alpha);
+      const int up_blocks = (ff + 127) / 128, down_blocks = (width + 255) / 256;
+      hipLaunchKernelGGL(moe_tile_kernel<true>, dim3(((size_t)max_tiles * up_blocks + 7) / 8 * 8), dim3(MOE_TILE_THREADS),
+                         MOE_TILE_LDS, s, (const bf16_t*)x, (const bf16_t*)w_gate_up, width, ff, tiles, max_tiles, places,
+                         top, (bf16_t*)hidden, (float*)nullptr, act, limit, alpha, up_blocks);
+      hipLaunchKernelGGL(moe_tile_kernel<false>, dim3(((size_t)max_tiles * down_blocks + 7) / 8 * 8), dim3(MOE_TILE_THREADS),
+                         MOE_TILE_LDS, s, (const bf16_t*)hidden, (const bf16_t*)w_down, ff, width, tiles, max_tiles, places,
+                         top, (bf16_t*)nullptr, y, act, limit, alpha, down_blocks);
     } else {
 #define QIL_MOE(T, MT, ALIGNED)                                                                                       \
   do {                                                                                                                \

@@ -50,8 +50,10 @@ class Attention(Mixer):
             raise ValueError('softcap must be positive')
         if type(self.value_dim) is not int or self.value_dim < 1:
             raise ops.UnsupportedShape(f'value_dim {self.value_dim!r} must be a positive integer')
-        if head_dim < 2 or head_dim % 2:
-            raise ops.UnsupportedShape(f'head_dim {head_dim} must be even')
+        rotated = getattr(position, 'rot_dim', 0) if position is not None else 0
+        if type(head_dim) is not int or head_dim < 1 or rotated > head_dim or (value_dim is None and head_dim % 2):
+            raise ops.UnsupportedShape(f'head_dim {head_dim} must be even (any size of at least the rotated width when '
+                                       'the values have a size of their own)')
         self.padded_dim = -(-max(head_dim, self.value_dim) // 8) * 8    # what the kernels and the cache see
         ops.check_attention_geometry(heads=heads, kv_heads=kv_heads, head_dim=self.padded_dim, dtype=dtype)
 

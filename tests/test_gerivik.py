@@ -304,6 +304,11 @@ ALONE = {
     'attention-values-narrower': plain.make_config(
         [plain.attention_layer(heads=9, kv_heads=3, dim=36, vdim=4, rot_dims=36, scale=0.02, softcap=100.0, base=20.0)],
         vocab=40, width=36, scale=9.0),
+    'attention-odd-sizes': plain.make_config(
+        [plain.attention_layer(heads=3, kv_heads=3, dim=11, vdim=7, rot_dims=4, scale=0.6, softcap=4.0)], vocab=40, width=18),
+    'attention-uses-a-later-layer': plain.make_config(
+        [dict(plain.attention_layer(heads=2, kv_heads=2, dim=8, vdim=8, rot_dims=8, scale=0.5, softcap=9.0), weights_of=1),
+         plain.attention_layer(heads=2, kv_heads=2, dim=8, vdim=8, rot_dims=8, scale=0.5, softcap=9.0)], vocab=40, width=16),
     'memory': plain.make_config([plain.gla_layer(heads=3, dim=10, vdim=70, tau=2.0)], vocab=40, width=30, scale=0.3),
     'memory-one-head-long-keys': plain.make_config([plain.gla_layer(heads=1, dim=130, vdim=12, tau=64.0)], vocab=40, width=20),
     'memory-twice': plain.make_config([plain.gla_layer(heads=2, dim=8, vdim=8, tau=1.5), dict(plain.gla_layer(heads=2, dim=8, vdim=8, tau=1.5), weights_of=0)],
@@ -450,6 +455,7 @@ def test_config_round_trip_and_refusals():
                    dict(config, layers=[dict(layers[0], weights_of=0)]),
                    dict(config, layers=[layers[0], dict(layers[1], weights_of=0)]),
                    dict(config, layers=layers[:4] + [dict(layers[1], weights_of=3)]),
+                   dict(config, layers=layers[:4] + [dict(layers[1], weights_of=7)]),
                    dict(config, layers=[dict(layers[0], mlp=plain.moe_mlp(ff=8, limit=1.0, experts=5, identity=2, top=2, count=2, keep=1))]),
                    dict(config, layers=[dict(layers[0], mlp=plain.moe_mlp(ff=8, limit=1.0, experts=4, identity=2, top=4, count=3, keep=1))])):
         with pytest.raises(ConfigError):
