@@ -229,10 +229,10 @@ def gerivik_config(z, layers, vocab):
     ffn = dict(kind='moe', expert=dict(ff=z['ff'] // 4, limit=7.0),
                router=dict(experts=30, identity=2, top=4, groups=dict(count=4, keep=2)))
     kinds = [
-        dict(type='gla', mlp=ffn, mixer=dict(heads=z['memory_heads'], dim=z['memory_dim'], vdim=z['memory_vdim'], tau=16.0)),
+        dict(type='gla', mlp=ffn, mixer=dict(heads=z['memory_heads'], dim=z['memory_dim'], vdim=z['memory_vdim'], tau=8.0)),
         dict(type='attention', mlp=ffn,
              mixer=dict(heads=z['heads'], kv_heads=max(1, z['heads'] // 4), dim=z['dim'], vdim=z['dim'],
-                        rot=dict(base=10000.0, dims=z['rot_dim']), scale=z['dim'] ** -0.5, softcap=50.0)),
+                        rot=dict(base=10000.0, dims=z['rot_dim']), scale=z['dim'] ** -0.5, softcap=30.0)),
     ]
     return dict(architecture='Gerivik', vocab=vocab, width=z['width'], embedding=dict(scale=1.0),
                 layers=[kinds[i % 2] for i in range(layers)], norm=dict(eps=1e-6))

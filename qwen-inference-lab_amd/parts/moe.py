@@ -52,9 +52,6 @@ class RoutedExperts(FeedForward):
             specs[f'experts.{e}.down_proj.weight'] = ParamSpec((self.width, self.intermediate))
         return specs
 
-    def param_names(self):
-        return list(self.param_specs())
-
     def finalize(self):
         p = self.p
         ff, padded = self.intermediate, -(-self.intermediate // 16) * 16
