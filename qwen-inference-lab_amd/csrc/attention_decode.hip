@@ -40,8 +40,9 @@ struct FusedQKV {
   const float* k_weight;
   float eps;
   const float* cos_table;                                  // null: no rotation
-  const float* sin_table;
+  const float* sin_table;                                  // null with a cos_table: that holds rot / 2 frequencies
   int rot;
+  int rotate_first;                                        // the rotation comes before the head norm
   int writes;                                              // 0: the cache belongs to another layer, which wrote it
 };
 
@@ -233,14 +234,16 @@ attn_decode_kernel(FusedQKV fused, const bf16_t* __restrict__ q, int q_stride, c
         float x[8];
         const int head = kvh * g + min(base + sub, g - 1);   // lanes past the group repeat its last head
         load8_sum_wide(fused.qkv, ((size_t)row * total_heads + head) * DMAX + chunk * 8, fused.splits, fused.split_stride, x);
-        norm_rope8<bf16_t>(x, chunk, TG, fused.q_weight, DMAX, fused.eps, fused.cos_table, fused.sin_table, pos, fused.rot);
+        norm_rope8<bf16_t>(x, chunk, TG, fused.q_weight, DMAX, fused.eps, fused.cos_table, fused.sin_table, pos, fused.rot,
+                           fused.rotate_first != 0);
         if (base + sub < g) shared_q[(base + sub) * TG + chunk] = pack8(x);
       }
       owner = fused.writes && pos >= begin && pos < end && wave == ((pos >> 5) - first_step) % waves;
       if (owner) {                                           // wave-uniform
         float x[8];
         load8_sum_wide(fused.qkv, ((size_t)row * total_heads + heads + kvh) * DMAX + chunk * 8, fused.splits, fused.split_stride, x);
-        norm_rope8<bf16_t>(x, chunk, TG, fused.k_weight, DMAX, fused.eps, fused.cos_table, fused.sin_table, pos, fused.rot);
+        norm_rope8<bf16_t>(x, chunk, TG, fused.k_weight, DMAX, fused.eps, fused.cos_table, fused.sin_table, pos, fused.rot,
+                           fused.rotate_first != 0);
         new_k = pack8(x);
         load8_sum_wide(fused.qkv, ((size_t)row * total_heads + heads + kv_heads + kvh) * DMAX + chunk * 8, fused.splits,
                        fused.split_stride, x);
@@ -410,19 +413,20 @@ extern "C" int qil_attn_decode_fused_takes(int heads, int kv_heads, int d, int p
 
 // qil_attn_decode with qkv [splits][rows][(heads + 2 kv_heads) d] float32 partial sums in the place of q; the
 // rows are the step's rows 0 .. rows-1 (no row index).  q_weight, k_weight: both or neither; cos/sin: both
-// or neither, [positions][rot / 2].  writes != 0: the new keys and values go into the caches at the rows'
+// [positions][rot / 2], or neither, or a cos_table alone that holds the rot / 2 frequencies (the angles are then made
+// in the kernel).  rotate_first: rotate, then norm.  softcap > 0: scores are capped softly after the scale.  writes != 0: the new keys and values go into the caches at the rows'
 // positions (the page comes from the block table).
 extern "C" int qil_attn_decode_fused(const float* qkv, int splits, const float* q_weight, const float* k_weight,
                                      float eps, const float* cos_table, const float* sin_table, int rot, int writes,
                                      void* k_cache, void* v_cache, const int* block_tables, int table_stride,
                                      const int* row_seq, const int* positions, void* workspace, void* out, int rows,
                                      int heads, int kv_heads, int d, int page_size, int window, float scale, int P,
-                                     int parts, int waves, int pairs, hipStream_t s) {
+                                     int parts, int waves, int pairs, int rotate_first, float softcap,
+                                     hipStream_t s) {
   if (rows == 0) return 0;
-  const float softcap = 0.f;                                 // (a capped attention makes its queries in qk_rope.hip)
   if (!qil_attn_decode_fused_takes(heads, kv_heads, d, page_size, cos_table ? rot : 0) || P % 32 || P < 32 ||
       parts < 1 || parts > 65535 || kv_heads > 65535 || waves < 1 || waves > DEC_MAX_WAVES || splits < 1 ||
-      (q_weight == nullptr) != (k_weight == nullptr) || (cos_table == nullptr) != (sin_table == nullptr) ||
+      (q_weight == nullptr) != (k_weight == nullptr) || (sin_table != nullptr && cos_table == nullptr) ||
       (((uintptr_t)qkv | (uintptr_t)q_weight | (uintptr_t)k_weight | (uintptr_t)cos_table | (uintptr_t)sin_table |
         (uintptr_t)k_cache) % 16))
     return -1;
@@ -438,6 +442,7 @@ extern "C" int qil_attn_decode_fused(const float* qkv, int splits, const float* 
   fused.splits = splits;
   fused.q_weight = q_weight; fused.k_weight = k_weight; fused.eps = eps;
   fused.cos_table = cos_table; fused.sin_table = sin_table; fused.rot = cos_table ? rot : 0;
+  fused.rotate_first = rotate_first;
   fused.writes = writes;
   const void* q = nullptr;
   const int q_stride = 0;

@@ -600,18 +600,18 @@ def decode_attention_takes(qkv, *, heads, kv_heads, head_dim, page_size, rotatio
     """Whether ``decode_attention`` takes the step: a float32 ``Partials`` q/k/v product, bfloat16 caches, sizes of
     the fused kernel."""
     rot = rotation.rot_dim if rotation is not None else 0
-    if rotation is not None and getattr(rotation, 'frequencies', None) is not None:
-        return False                                   # (the fused kernel rotates from tables)
     return isinstance(qkv, Partials) and qkv.shape[0] <= FUSED_DECODE_MOST_ROWS and dtype == torch.bfloat16 and \
         bool(library.load().qil_attn_decode_fused_takes(heads, kv_heads, head_dim, page_size, rot))
 
 
 def decode_attention(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps, rotation, positions, writes, k_cache,
-                     v_cache, page_size, block_tables, row_seq, max_context, scale, window, unmerged=False):
+                     v_cache, page_size, block_tables, row_seq, max_context, scale, window, unmerged=False,
+                     rotate_first=False, softcap=None):
     """``qk_norm_rope_store`` and ``paged_attention`` in one kernel for a step whose rows are all alone in their
     sequences: queries, the new key and the new value are made from the partial sums ``qkv`` inside the
     attention kernel (bit for bit what the two kernels make), the new key and value are written into the
-    pages (``writes``) and used from registers.  Returns what ``paged_attention`` returns."""
+    pages (``writes``) and used from registers.  ``rotate_first`` and ``softcap`` as in ``qk_norm_rope_store`` and
+    ``paged_attention``.  Returns what ``paged_attention`` returns."""
     n = qkv.shape[0]
     dtype = torch.bfloat16
     _require(qkv.tensor, 'qkv', torch.float32, (qkv.splits, n, (heads + 2 * kv_heads) * head_dim))
@@ -624,14 +624,7 @@ def decode_attention(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps,
     for w, name in ((q_weight, 'q_weight'), (k_weight, 'k_weight')):
         if w is not None:
             _require(w, name, torch.float32, (head_dim,))
-    cos = sin = None
-    rot = 0
-    if rotation is not None:
-        cos, sin, rot = rotation.cos, rotation.sin, rotation.rot_dim
-        _require(cos, 'cos', torch.float32)
-        _require(sin, 'sin', torch.float32, cos.shape)
-        if cos.shape[1] * 2 != rot or rot > head_dim:
-            raise ValueError('rotation tables do not fit rot_dim')
+    cos, sin, rot = _rotation_arguments(rotation, head_dim)
     lib = library.load()
     out = torch.empty((n, heads * head_dim), dtype=dtype, device=k_cache.device)
     window_arg = int(window or 0)
@@ -643,7 +636,7 @@ def decode_attention(qkv, *, heads, kv_heads, head_dim, q_weight, k_weight, eps,
                                      block_tables.shape[1], _ptr(row_seq), _ptr(positions), _ptr(workspace), _ptr(out),
                                      n, heads, kv_heads, head_dim, page_size, window_arg, float(scale), part, parts,
                                      DECODE_WAVES, int(n * kv_heads * parts <= DECODE_PAIRS_BLOCKS and head_dim <= FUSED_PAIRS_MOST_DIM),
-                                     _stream()), 'attn_decode_fused')
+                                     int(bool(rotate_first)), float(softcap or 0.0), _stream()), 'attn_decode_fused')
     if parts > 1:
         result = Unmerged(workspace, positions, out, heads=heads, head_dim=head_dim, window=window_arg, part=part,
                           parts=parts)

@@ -121,16 +121,15 @@ class Attention(Mixer):
             norms = dict(q_weight=p.get('q_norm.weight'), k_weight=p.get('k_norm.weight'),
                          eps=self.qk_norm_eps if self.qk_norm_eps is not None else 0.0)
         sizes = dict(heads=self.heads, kv_heads=self.kv_heads, head_dim=self.padded_dim)
-        # (the kernel that makes its queries itself norms over the whole head it sees, norms before it rotates and
-        # caps nothing: not for padded heads, and not for designs that differ there)
-        if ctx.max_query == 1 and self.padded_dim == self.head_dim and self.softcap is None and \
-                not self.norm_after_rotation and \
+        # (the kernel that makes its queries itself norms over the whole head it sees: not for padded heads)
+        if ctx.max_query == 1 and self.padded_dim == self.head_dim and \
                 ops.decode_attention_takes(qkv, page_size=cache.page_size, rotation=rotation, dtype=self.dtype, **sizes):
             # every row alone in its sequence: norm, rotation and cache write happen inside the attention kernel
             attended = ops.decode_attention(
                 qkv, rotation=rotation, positions=ctx.positions, writes=cache.writes, k_cache=cache.k, v_cache=cache.v,
                 page_size=cache.page_size, block_tables=cache.block_tables, row_seq=ctx.row_seq,
-                max_context=ctx.max_context, scale=self.scale, window=self.window, unmerged=True, **sizes, **norms)
+                max_context=ctx.max_context, scale=self.scale, window=self.window, unmerged=True,
+                rotate_first=self.norm_after_rotation, softcap=self.softcap, **sizes, **norms)
             return ops.linear(attended, p['o_proj.weight'], p.get('o_proj.bias'), partials=True)
         q = ops.qk_norm_rope_store(
             qkv, rotation=rotation, positions=ctx.positions, slots=cache.slots if cache.writes else None,

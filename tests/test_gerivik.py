@@ -304,6 +304,9 @@ ALONE = {
     'attention-values-narrower': plain.make_config(
         [plain.attention_layer(heads=9, kv_heads=3, dim=36, vdim=4, rot_dims=36, scale=0.02, softcap=100.0, base=20.0)],
         vocab=40, width=36, scale=9.0),
+    'attention-heads-of-64': plain.make_config(                   # (sizes of the decode kernel that makes its own queries)
+        [plain.attention_layer(heads=4, kv_heads=2, dim=64, vdim=64, rot_dims=32, scale=0.2, softcap=6.0),
+         plain.attention_layer(heads=2, kv_heads=1, dim=128, vdim=64, rot_dims=64, scale=0.1, softcap=15.0)], vocab=40, width=64),
     'attention-odd-sizes': plain.make_config(
         [plain.attention_layer(heads=3, kv_heads=3, dim=11, vdim=7, rot_dims=4, scale=0.6, softcap=4.0)], vocab=40, width=18),
     'attention-uses-a-later-layer': plain.make_config(

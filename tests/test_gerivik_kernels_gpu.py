@@ -145,6 +145,50 @@ def test_capped_scores_in_decoding_and_in_prompts(dtype, lengths, page_size, d, 
     close(got, want, dtype)
 
 
+@pytest.mark.parametrize('lengths,page_size,d,heads,kv_heads,rot,splits,cap', [
+    ([1, 2, 31, 32, 33, 64, 65, 96], 8, 64, 6, 2, 32, 3, 0.5),
+    ([2100, 1, 700, 1290, 64, 2047, 300, 33], 16, 128, 16, 4, 64, 8, 30.0),
+    ([257, 512, 513], 32, 128, 8, 1, 128, 1, 5.0),
+])
+def test_decoding_with_queries_made_inside_is_the_two_kernels(lengths, page_size, d, heads, kv_heads, rot, splits, cap):
+    """The decode kernel that makes queries, the new key and the new value itself, with the rotation from frequencies
+    before a unit norm and capped scores: bit for bit what the q/k kernel followed by the attention kernel leave."""
+    dtype = torch.bfloat16
+    rows, total = len(lengths), heads + 2 * kv_heads
+    k_cache, v_cache, table, _ = build_cache(lengths, page_size, kv_heads, d, dtype)
+    positions = torch.tensor([n - 1 for n in lengths], dtype=torch.int32).cuda()
+    row_seq = torch.arange(rows, dtype=torch.int32).cuda()
+    slots = (table[row_seq.long(), (positions // page_size).long()] * page_size + positions % page_size).to(torch.int32)
+    g = torch.Generator().manual_seed(d)
+    qkv = ops.Partials((torch.randn(splits, rows, total * d, generator=g) * 0.7).cuda())
+    ones = torch.ones(d).cuda()
+    frequencies = torch.tensor([5000.0 ** (-2 * i / rot) for i in range(rot // 2)], dtype=torch.float32).cuda()
+    rotation = Rotation(None, None, rot, frequencies)
+    sizes = dict(heads=heads, kv_heads=kv_heads, head_dim=d)
+    assert ops.decode_attention_takes(qkv, page_size=page_size, rotation=rotation, dtype=dtype, **sizes)
+    k_two, v_two = k_cache.clone(), v_cache.clone()
+    q = ops.qk_norm_rope_store(qkv, q_weight=ones, k_weight=ones, eps=1e-6, rotation=rotation, positions=positions,
+                               slots=slots, k_cache=k_two, v_cache=v_two, page_size=page_size, dtype=dtype,
+                               rotate_first=True, **sizes)
+    want = ops.paged_attention(q, k_cache=k_two, v_cache=v_two, page_size=page_size, block_tables=table, row_seq=row_seq,
+                               positions=positions, cu_seqlens=None, seq_starts=None, single_rows=None, n_seqs=rows,
+                               max_query=1, max_context=max(lengths), scale=2.0 * d ** -0.5, window=None, softcap=cap, **sizes)
+    k_one, v_one = k_cache.clone(), v_cache.clone()
+    got = ops.decode_attention(qkv, q_weight=ones, k_weight=ones, eps=1e-6, rotation=rotation, positions=positions,
+                               writes=True, k_cache=k_one, v_cache=v_one, page_size=page_size, block_tables=table,
+                               row_seq=row_seq, max_context=max(lengths), scale=2.0 * d ** -0.5, window=None,
+                               rotate_first=True, softcap=cap, **sizes)
+    assert torch.isfinite(got.float()).all()
+    torch.testing.assert_close(got, want, atol=0, rtol=0)
+    same = lambda a, b: torch.equal(a.view(torch.int16), b.view(torch.int16))          # NaN-filled pages: compare the bits
+    assert same(k_one, k_two) and same(v_one, v_two), 'the pages differ'
+    uncapped = ops.decode_attention(qkv, q_weight=ones, k_weight=ones, eps=1e-6, rotation=rotation, positions=positions,
+                                    writes=False, k_cache=k_one, v_cache=v_one, page_size=page_size, block_tables=table,
+                                    row_seq=row_seq, max_context=max(lengths), scale=2.0 * d ** -0.5, window=None,
+                                    rotate_first=True, softcap=None, **sizes)
+    assert not torch.equal(uncapped, got)
+
+
 # ------------------------------------------------------------------------------------------------ the memory's decays
 @pytest.mark.parametrize('dtype', DTYPES)
 @pytest.mark.parametrize('sizes', [dict(heads=2, dim=24, vdim=16), dict(heads=3, dim=72, vdim=130),
