@@ -527,7 +527,8 @@ int qil_moe_max_tiles(int pairs, int experts, int tile_rows) { return (pairs + t
 
 // The experts' work on the routed pairs: x [n, width], chosen/weights [n, top]; w_gate_up [experts][2][ff][width],
 // w_down [experts][width][ff] (dtype); scratch: tiles int32 [3 * max_tiles], places int32 [n * top], hidden (dtype)
-// [n * top, ff], y float32 [n * top, width].  out float32 [n, width].
+// [n * top, ff], y float32 [n * top, width].  out float32 [n, width], or null: the pairs' rows stay in y for a consumer
+// that makes the weighted sum itself.
 int qil_moe_experts(const void* x, int dtype, const int* chosen, const float* weights, const void* w_gate_up,
                     const void* w_down, int* tiles, int* places, void* hidden, float* y, float* out, int n, int width,
                     int ff, int experts, int top, int tile_rows, int max_tiles, int act, float limit, float alpha,
@@ -577,6 +578,21 @@ int qil_moe_experts(const void* x, int dtype, const int* chosen, const float* we
 #undef QIL_MOE
     }
   }
+  if (!out) QIL_RETURN_LAUNCH_STATUS();                  // the caller's next norm makes the weighted sum itself
+  const int threads = width >= 1024 ? 256 : 64;
+  if (dtype == QIL_F32)
+    hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(n), dim3(threads), 0, s, (const float*)x, y, chosen, weights,
+                       experts, top, width, out);
+  else
+    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, dim3(n), dim3(threads), 0, s, (const bf16_t*)x, y, chosen, weights,
+                       experts, top, width, out);
+  QIL_RETURN_LAUNCH_STATUS();
+}
+
+// The weighted sum alone (what qil_moe_experts ends with when it is given an `out`).
+int qil_moe_combine(const void* x, int dtype, const float* y, const int* chosen, const float* weights, float* out, int n,
+                    int width, int experts, int top, hipStream_t s) {
+  if (n == 0) return 0;
   const int threads = width >= 1024 ? 256 : 64;
   if (dtype == QIL_F32)
     hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(n), dim3(threads), 0, s, (const float*)x, y, chosen, weights,

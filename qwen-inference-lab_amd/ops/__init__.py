@@ -162,12 +162,52 @@ class PostNormed:
         self.shape, self.device = tuple(value.shape), value.device
 
 
+class RoutedSum:
+    """The result of a routed feed-forward before its weighted sum: ``pairs`` float32 [N * top, width] (every (token,
+    slot) pair's expert output), ``weights`` and ``chosen`` [N, top], and the feed-forward's input ``x`` (what an
+    identity expert, a chosen index from ``experts`` on, passes).  A norm that takes a ``PostNormed`` makes the sum
+    while it loads the row; ``materialize()`` runs the sum's own kernel."""
+
+    def __init__(self, x, pairs, chosen, weights, experts):
+        self.x, self.pairs, self.chosen, self.weights, self.experts = x, pairs, chosen, weights, int(experts)
+        self.shape, self.device, self.dtype = tuple(x.shape), x.device, x.dtype
+
+    def materialize(self):
+        n, width = self.shape
+        out = torch.empty((n, width), dtype=torch.float32, device=self.device)
+        _check(library.load().qil_moe_combine(_ptr(self.x), _code(self.dtype), _ptr(self.pairs), _ptr(self.chosen),
+                                              _ptr(self.weights), _ptr(out), n, width, self.experts, self.chosen.shape[1],
+                                              _stream()), 'moe_combine')
+        return out
+
+
+def _plain_delta(delta):
+    """A pending sub-layer output as the norms' kernels take it: a routed sum is made first."""
+    return Partials(delta.materialize().unsqueeze(0)) if isinstance(delta, RoutedSum) else delta
+
+
 def _post_normed(stream, pending, rows, weight, eps, out_dtype, update):
     n, width = stream.shape
     value = pending.value
     _require(stream, 'stream', torch.float32)
     _require(weight, 'weight', torch.float32, (width,))
     _require(pending.weight, 'post-norm weight', torch.float32, (width,))
+    if isinstance(value, RoutedSum) and value.dtype == out_dtype:
+        top = value.chosen.shape[1]
+        _require(value.x, 'routed input', out_dtype, (n, width))
+        _require(value.pairs, 'routed pairs', torch.float32, (n * top, width))
+        _require(value.chosen, 'chosen', torch.int32, (n, top))
+        _require(value.weights, 'weights', torch.float32, (n, top))
+        if rows is not None:
+            _require(rows, 'rows', torch.int32)
+        count = n if rows is None else rows.shape[0]
+        out = torch.empty((count, width), dtype=out_dtype, device=stream.device)
+        _check(library.load().qil_post_norm_add_norm_routed(
+            _ptr(stream), _ptr(value.pairs), _ptr(value.weights), _ptr(value.chosen), _ptr(value.x), top, value.experts,
+            _ptr(pending.weight), pending.eps, _ptr(rows), _ptr(weight), _ptr(out), count, width, float(eps), int(update),
+            _code(out_dtype), _stream()), 'post_norm_add_norm_routed')
+        return out
+    value = _plain_delta(value)
     if isinstance(value, Partials):
         _require(value.tensor, 'delta', torch.float32, (value.splits, n, width))
         pointer, code, splits = value.tensor.data_ptr(), 0, value.splits
@@ -276,6 +316,7 @@ def add_rmsnorm(stream, delta, weight, eps, out_dtype):
     ``delta``: tensor of ``out_dtype`` [N, H], Partials, or a ``PostNormed`` (its norm is what is added)."""
     if isinstance(delta, PostNormed):
         return _post_normed(stream, delta, None, weight, eps, out_dtype, True)
+    delta = _plain_delta(delta)
     n, width = stream.shape
     _require(stream, 'stream', torch.float32)
     _require(weight, 'weight', torch.float32, (width,))
@@ -290,6 +331,7 @@ def rows_rmsnorm(stream, delta, rows, weight, eps, out_dtype):
     """norm(stream[rows] + delta[rows]) as out_dtype [len(rows), H]; stream is left as it is."""
     if isinstance(delta, PostNormed):
         return _post_normed(stream, delta, rows, weight, eps, out_dtype, False)
+    delta = _plain_delta(delta)
     n, width = stream.shape
     _require(stream, 'stream', torch.float32)
     _require(weight, 'weight', torch.float32, (width,))
@@ -1112,8 +1154,9 @@ def moe_route(x, router, correction, *, groups, keep, top, renormalize=False):
     return chosen, weights
 
 
-def moe_experts(x, chosen, weights, gate_up, down, *, activation, limit=0.0, alpha=1.0):
-    """The weighted sum of the chosen experts' outputs, float32 [N, width].  ``gate_up`` [experts, 2, ff, width] (an
+def moe_experts(x, chosen, weights, gate_up, down, *, activation, limit=0.0, alpha=1.0, lazy=False):
+    """The weighted sum of the chosen experts' outputs, float32 [N, width]; with ``lazy`` a ``RoutedSum`` (the pairs'
+    rows, for a norm that makes the sum while it loads them).  ``gate_up`` [experts, 2, ff, width] (an
     expert's gate rows, then its up rows), ``down`` [experts, width, ff], both of x's type; an expert computes
     down(act(gate x, up x)) with ``activation`` of ``GATE_FUNCTIONS``.  A chosen index from ``experts`` on is an
     identity expert: its output is x itself.  The pairs (token, chosen expert) are grouped by expert on the device;
@@ -1133,9 +1176,9 @@ def moe_experts(x, chosen, weights, gate_up, down, *, activation, limit=0.0, alp
     scratch = torch.empty(3 * max_tiles + pairs, dtype=torch.int32, device=x.device)
     hidden = torch.empty((pairs, ff), dtype=x.dtype, device=x.device)
     y = torch.empty((pairs, width), dtype=torch.float32, device=x.device)
-    out = torch.empty((n, width), dtype=torch.float32, device=x.device)
+    out = None if lazy else torch.empty((n, width), dtype=torch.float32, device=x.device)
     _check(lib.qil_moe_experts(_ptr(x), _code(x.dtype), _ptr(chosen), _ptr(weights), _ptr(gate_up), _ptr(down),
                                _ptr(scratch), scratch[3 * max_tiles:].data_ptr(), _ptr(hidden), _ptr(y), _ptr(out), n, width,
                                ff, experts, top, tile_rows, max_tiles, GATE_FUNCTIONS[activation], float(limit),
                                float(alpha), _stream()), 'moe_experts')
-    return out
+    return RoutedSum(x, y, chosen, weights, experts) if lazy else out

@@ -319,6 +319,10 @@ def _declare(lib):
         getattr(lib, name).restype = i
     lib.qil_post_norm_add_norm.argtypes = [p, p, i, i, i, p, f, p, p, p, i, i, f, i, i, p]
     lib.qil_post_norm_add_norm.restype = i
+    lib.qil_post_norm_add_norm_routed.argtypes = [p, p, p, p, p, i, i, p, f, p, p, p, i, i, f, i, i, p]
+    lib.qil_post_norm_add_norm_routed.restype = i
+    lib.qil_moe_combine.argtypes = [p, i, p, p, p, p, i, i, i, i, p]
+    lib.qil_moe_combine.restype = i
     lib.qil_moe_takes.argtypes = [i, i, i, i, i, i]
     lib.qil_moe_takes.restype = i
     lib.qil_moe_route.argtypes = [p, i, p, p, p, p, p, i, i, i, i, i, i, i, p]

@@ -69,5 +69,7 @@ class RoutedExperts(FeedForward):
         chosen, weights = ops.moe_route(h, p['router.weight'], p.get('router.correction'), groups=self.groups,
                                         keep=self.keep, top=self.top, renormalize=self.renormalize)
         out = ops.moe_experts(h, chosen, weights, p['experts.gate_up_proj.weight'], p['experts.down_proj.weight'],
-                              activation=self.activation, limit=self.limit, alpha=self.alpha)
+                              activation=self.activation, limit=self.limit, alpha=self.alpha, lazy=True)
+        if isinstance(out, ops.RoutedSum):              # the norm that follows makes the weighted sum as it loads the rows
+            return out
         return ops.Partials(out.unsqueeze(0))           # complete float32 sums: one split

@@ -342,7 +342,7 @@ def moe_route(x, router, correction, *, groups, keep, top, renormalize=False):
     return chosen.to(torch.int32), weights
 
 
-def moe_experts(x, chosen, weights, gate_up, down, *, activation, limit=0.0, alpha=1.0):
+def moe_experts(x, chosen, weights, gate_up, down, *, activation, limit=0.0, alpha=1.0, lazy=False):
     """float32 [N, width]; the hidden activations pass through x's type as the kernel's do."""
     n, width = x.shape
     experts = gate_up.shape[0]

@@ -316,6 +316,15 @@ def test_the_experts_against_the_reference(dtype, sizes):
     got = ops.moe_experts(x.cuda(), chosen.cuda(), weights.cuda(), gate_up.cuda(), down.cuda(), **act)
     want = refs.moe_experts(x, chosen, weights, gate_up, down, **act)
     close(got, want, dtype, max(1.0, want.abs().max().item()))
+    # left for the next norm to sum: the same numbers through the norm's kernel as through the sum's own
+    lazy = ops.moe_experts(x.cuda(), chosen.cuda(), weights.cuda(), gate_up.cuda(), down.cuda(), lazy=True, **act)
+    close(lazy.materialize(), want, dtype, max(1.0, want.abs().max().item()))
+    stream, post, weight = torch.randn(n, width, generator=g), 1 + 0.1 * torch.randn(width, generator=g), torch.ones(width)
+    through = [s.clone().cuda() for s in (stream, stream)]
+    one = ops.add_rmsnorm(through[0], ops.PostNormed(lazy, post.cuda(), 1e-6), weight.cuda(), 1e-6, dtype)
+    two = ops.add_rmsnorm(through[1], ops.PostNormed(got, post.cuda(), 1e-6), weight.cuda(), 1e-6, dtype)
+    close(through[0], through[1].cpu(), torch.float32)
+    close(one, two.cpu(), dtype)
     # a token's result does not depend on who else is in the step
     alone = ops.moe_experts(x[:1].cuda(), chosen[:1].cuda(), weights[:1].cuda(), gate_up.cuda(), down.cuda(), **act)
     assert torch.equal(alone[0], got[0])
@@ -332,7 +341,7 @@ def test_the_routed_part_against_experts_one_by_one():
         part.set_param(name, t.cuda())
     part.finalize()
     h = torch.randn(n, width, generator=g)
-    out = part.forward(h.cuda()).sum().cpu()
+    out = part.forward(h.cuda()).materialize().cpu()
     s = torch.softmax(h @ tensors['router.weight'].t(), dim=-1)
     choice = s + tensors['router.correction']
     group = choice.view(n, 2, 2).max(-1).values.argmax(-1)
